@@ -1,0 +1,87 @@
+/*
+ * msgl_mix.h -- C ABI of the sequence-mixing kernels (latent attention, linear-recurrence layers, routed experts)
+ * for gfx950; implemented by libmsgl_mix.so (mini-sglang_amd/csrc/seqmix.hip).
+ *
+ * Same conventions as msgl_hip.h: raw device pointers, explicit sizes and strides in ELEMENTS, `stream` is a
+ * hipStream_t passed as void*, every function returns 0 or a negative code and leaves a message for
+ * msgl_mix_last_error(); nothing allocates, frees or synchronises, so every call may be captured in a hipGraph.
+ * `dtype` is the model dtype T of the tensors that feed matrix products (bf16 or fp32); the residual stream, norms,
+ * scores, recurrent state and router are fp32 whatever T is.
+ */
+#ifndef MSGL_MIX_H_
+#define MSGL_MIX_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MSGL_MIX_OK 0
+#define MSGL_MIX_EINVAL (-1)
+#define MSGL_MIX_ELAUNCH (-2)
+
+#define MSGL_MIX_BF16 0
+#define MSGL_MIX_F32 2
+
+#define MSGL_MIX_ACT_NONE 0
+#define MSGL_MIX_ACT_RELU2 1 /* max(z, 0)^2 */
+
+#define MSGL_MIX_ABI_VERSION 1
+
+const char* msgl_mix_last_error(void);
+int msgl_mix_abi_version(void);
+
+/* x32[t] = table[ids[t]] as fp32, h[t] = the same row in T. */
+int msgl_mix_embed(float* x32, void* h, const void* table, const int* ids, int tokens, int W, int dtype, void* stream);
+
+/* s = alpha * x_in + sum_p gate[t, p] * y[t, p]   (y: [rows, parts, W] in T or null with parts = 0; gate: fp32 [rows, parts] or
+ * null = ones);   out = s / sqrt(mean(s^2) + eps) * (1 + w).  Written to x_out (fp32, may alias x_in) and / or h_out (T). */
+int msgl_mix_postnorm(const float* x_in, float* x_out, void* h_out, const void* y, int parts, const float* gate, const void* w,
+                      float alpha, float eps, int rows, int W, int dtype, void* stream);
+
+/* One projection row per token = [q: H x (d + r) | latent R | shared rotated key part r] (the last two only with has_kv).
+ * Writes the rotated query parts into q_abs[t, h, R : R + r] (fp32, rows of R + r) and, with has_kv, the RMS-normed latent
+ * (plain weight c_norm_w) and the rotated key part into cache[out_loc[t]] (rows of R + r, T).
+ * cos_sin: fp32 [positions, rot_dims] = cos | sin halves; entries rot_dims .. r of a rotated part pass unchanged. */
+int msgl_mix_latent_prep(const void* proj, int64_t ld_proj, float* q_abs, void* cache, const int* out_loc, const int* positions,
+                         const float* cos_sin, const void* c_norm_w, float eps, int tokens, int H, int d, int r, int rot_dims, int R,
+                         int has_kv, int dtype, void* stream);
+
+/* Causal attention of H heads over ONE shared key row per token: score = q_abs[t, h] . cache[slot] * scale over dk entries,
+ * softmax in fp32, out[t, h] = sum_j p_j cache[slot_j][0 : dv] (fp32).  Requests as in the paged backend: table rows of token
+ * slots, seq_lens = keys after this forward, cu_q = exclusive prefix of new tokens; prefill portions, single decoded tokens
+ * and any mix of them in one launch. */
+int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, const int* table, int64_t table_stride, const int* req_rows,
+                         const int* seq_lens, const int* cu_q, int batch, int total_q, int H, int dk, int dv, float scale, int dtype,
+                         void* stream);
+
+/* Linear recurrence per (request, head): S <- decay[h] S + k v^T, out = S^T q, with q, k, v = SiLU of the projection row
+ * [q: H x d | k: H x d | v: H x dv | ...].  state: fp32 [slots, H, d, dv], row slots[b]; a request whose first new token is at
+ * position 0 (seq_lens[b] == its new tokens) starts from zero.  out: fp32 [tokens, H * dv]. */
+int msgl_mix_lightning(float* out, const void* qkv, int64_t ld_qkv, float* state, const float* decay, const int* cu_q, const int* seq_lens,
+                       const int* slots, int batch, int H, int d, int dv, int dtype, void* stream);
+
+/* out = o / sqrt(mean(o^2) + eps) * w * sigmoid(gate) over rows of N (o fp32, out and gate T). */
+int msgl_mix_gated_norm(void* out, const float* o, const void* gate, int64_t ld_gate, const void* w, float eps, int rows, int N, int dtype,
+                        void* stream);
+
+/* Router: s = softmax(router h) in fp32; choice = s + bias (bias may be null); only experts of the `keep` best of G equal
+ * groups of neighbours (group score = its largest choice) can win; ids = the `top` largest choices, wts = their s / (sum + 1e-20). */
+int msgl_mix_route(int* ids, float* wts, const void* h, const void* router, const void* bias, int tokens, int W, int E, int top, int G,
+                   int keep, int dtype, void* stream);
+
+/* seg[E + 1], perm[n]: flat (token, choice) indices bucketed by expert, stable inside a bucket. */
+int msgl_mix_moe_sort(int* seg, int* perm, const int* ids, int n, int E, void* stream);
+
+/* C[g] = act(A[g] B[g]^T) with fp32 accumulation; groups advance by *_gs elements.  With seg, group g owns rows
+ * seg[g] .. seg[g + 1] of one shared row space of at most M rows (A and C do not advance per group then); a_rows / c_rows
+ * make that row space indirect (A row = a_rows[m] / a_div, C row = c_rows[m]).  ta / tb / tc: dtype codes. */
+int msgl_mix_gemm_nt(void* C, const void* A, const void* B, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int groups,
+                     int64_t a_gs, int64_t b_gs, int64_t c_gs, const int* seg, const int* a_rows, int a_div, const int* c_rows, int act,
+                     int ta, int tb, int tc, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

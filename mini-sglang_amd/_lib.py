@@ -19,6 +19,8 @@ LIB_DIR = _PKG / "lib"
 HIP_SO = LIB_DIR / "libmsgl_hip.so"
 COMM_SO = LIB_DIR / "libmsgl_comm.so"
 GEMM_SO = LIB_DIR / "libmsgl_gemm.so"
+MIX_SO = LIB_DIR / "libmsgl_mix.so"
+MIX_ABI_VERSION = 1
 
 BF16, FP16, F32 = 0, 1, 2
 UNIQUE_ID_BYTES = 128
@@ -137,6 +139,22 @@ GEMM_SIGNATURES = {
 }
 
 
+# mirrors include/msgl_mix.h one to one
+MIX_SIGNATURES = {
+    "msgl_mix_last_error": (C.c_char_p, []),
+    "msgl_mix_abi_version": (_i, []),
+    "msgl_mix_embed": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
+    "msgl_mix_postnorm": (_i, [_p, _p, _p, _p, _i, _p, _p, _f, _f, _i, _i, _i, _p]),
+    "msgl_mix_latent_prep": (_i, [_p, _l, _p, _p, _p, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_latent_attn": (_i, [_p, _p, _p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _p]),
+    "msgl_mix_lightning": (_i, [_p, _p, _l, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_gated_norm": (_i, [_p, _p, _p, _l, _p, _f, _i, _i, _i, _p]),
+    "msgl_mix_route": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_moe_sort": (_i, [_p, _p, _p, _i, _i, _p]),
+    "msgl_mix_gemm_nt": (_i, [_p, _p, _p, _i, _i, _i, _l, _l, _l, _i, _l, _l, _l, _p, _p, _i, _p, _i, _i, _i, _i, _p]),
+}
+
+
 class MsglError(RuntimeError):
     """Raised when a C-ABI call returns a negative code (reference: host::PanicError)."""
 
@@ -195,6 +213,24 @@ def gemm_lib() -> C.CDLL:
     if _gemm is None:
         _gemm = _bind(GEMM_SO, GEMM_SIGNATURES)
     return _gemm
+
+
+_mix: C.CDLL | None = None
+
+
+def mix_lib() -> C.CDLL:
+    global _mix
+    if _mix is None:
+        _mix = _bind(MIX_SO, MIX_SIGNATURES)
+        if _mix.msgl_mix_abi_version() != MIX_ABI_VERSION:
+            raise RuntimeError("libmsgl_mix.so ABI version mismatch; rebuild")
+    return _mix
+
+
+def check_mix(rc: int, what: str = "") -> None:
+    if rc < 0:
+        msg = mix_lib().msgl_mix_last_error().decode(errors="replace")
+        raise MsglError(f"{what or 'msgl mix call'} failed ({rc}): {msg}")
 
 
 def check_gemm(rc: int, what: str = "") -> None:

@@ -211,3 +211,63 @@ class HipAttnBackend:
         self._cap_seq[:bs].copy_(md.seq_lens)
         self._cap_rows[:bs].copy_(md.req_rows)
         ops.attn_decode_plan(self._cap_plan, self._cap_seq, bs, self.max_bs, self.capacity, self.qo_heads, self.kv_heads)
+
+
+class MixAttnBackend:
+    """Batch metadata for the hybrid decoders (latent attention + linear recurrence): the same three vectors the paged
+    backend hands its kernels -- keys per request after this forward, page-table row, exclusive prefix of new tokens -- in
+    one pinned buffer and one asynchronous copy.  Their kernels take prompt portions, single decoded tokens and any mix of
+    the two in one launch, so there is no prefill / decode split and no work plan; the recurrent layers use the table row
+    as the request's state slot.  Graph capture keeps static copies of the vectors, refreshed before every replay."""
+
+    def __init__(self, config: Any, ctx: Any = None, *, tp_size: int = 1) -> None:
+        ctx = ctx if ctx is not None else _core.get_global_ctx()
+        self.ctx, self.config = ctx, config
+        self.kvcache = ctx.kv_cache
+        self.device = self.kvcache.device
+        self.max_bs = int(ctx.page_table.shape[0])
+        self.capture_bs: List[int] = []
+        self._cap: Optional[torch.Tensor] = None
+
+    def prepare_metadata(self, batch: Any) -> None:
+        reqs = batch.padded_reqs
+        bs = len(reqs)
+        q = np.fromiter((r.extend_len for r in reqs), dtype=np.int64, count=bs)
+        k = np.fromiter((r.device_len for r in reqs), dtype=np.int64, count=bs)
+        rows = np.fromiter((r.table_idx for r in reqs), dtype=np.int64, count=bs)
+        host = torch.empty(3 * bs + 1, dtype=torch.int32, pin_memory=True)
+        h = host.numpy()
+        h[:bs], h[bs: 2 * bs], h[2 * bs] = k, rows, 0
+        h[2 * bs + 1:] = np.cumsum(q)
+        dev = host.to(self.device, non_blocking=True)
+        batch.attn_metadata = HipAttnMetadata(cu_seqlens_q=dev[2 * bs:], seq_lens=dev[:bs], req_rows=dev[bs: 2 * bs], batch=bs,
+                                              max_seqlen_q=int(q.max()), max_seqlen_k=int(k.max()))
+
+    # ------------------------------------------------------------------ graph hooks
+    def init_capture_graph(self, max_seq_len: int, bs_list: List[int]) -> None:
+        assert self._cap is None, "Capture already initialized."
+        n = max(bs_list)
+        assert n <= self.max_bs
+        self.capture_bs = sorted(bs_list)
+        self._cap = torch.zeros(3 * n + 1, dtype=torch.int32, device=self.device)
+        self._cap_n = n
+
+    def _static(self, bs: int) -> HipAttnMetadata:
+        n, c = self._cap_n, self._cap
+        return HipAttnMetadata(cu_seqlens_q=c[2 * n: 2 * n + bs + 1], seq_lens=c[:bs], req_rows=c[n: n + bs], batch=bs,
+                               max_seqlen_q=1, max_seqlen_k=int(self.ctx.page_table.shape[1]))
+
+    def prepare_for_capture(self, batch: Any) -> None:
+        bs, n = batch.size, self._cap_n
+        assert bs in self.capture_bs
+        self._cap[:bs].fill_(1)
+        self._cap[n: n + bs].fill_(batch.reqs[0].table_idx)
+        self._cap[2 * n: 2 * n + bs + 1].copy_(torch.arange(bs + 1, dtype=torch.int32, device=self.device))
+        batch.attn_metadata = self._static(bs)
+
+    def prepare_for_replay(self, batch: Any) -> None:
+        md, bs, n = batch.attn_metadata, batch.padded_size, self._cap_n
+        assert bs in self.capture_bs
+        self._cap[:bs].copy_(md.seq_lens)
+        self._cap[n: n + bs].copy_(md.req_rows)
+        self._cap[2 * n: 2 * n + bs + 1].copy_(md.cu_seqlens_q)

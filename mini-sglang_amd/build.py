@@ -7,6 +7,9 @@ Outputs (git-ignored, shipped to the GPU box by gpurun because they are in-tree)
     mini-sglang_amd/lib/libmsgl_hip.so    every kernel + host helpers   (include/msgl_hip.h)
     mini-sglang_amd/lib/libmsgl_comm.so   RCCL communicator             (links librccl)
     mini-sglang_amd/lib/libmsgl_gemm.so   projection GEMMs + tuner      (links libhipblaslt)
+    mini-sglang_amd/lib/libmsgl_mix.so    sequence-mixing kernels       (include/msgl_mix.h; no library dependency)
+
+`build_all(only=("mix", "gemm"))` builds a subset: a model needs the libraries its layers call, not all of them.
 
 hipcc cross-compiles for gfx950 without a GPU, so this also runs in the build container.
 """
@@ -43,6 +46,7 @@ HIP_SOURCES = [
     "gemm_ro.hip",
     "comm_p2p.hip",
 ]
+MIX_SOURCES = ["seqmix.hip"]
 COMM_SOURCES = ["comm.cpp"]
 GEMM_SOURCES = ["gemm.cpp"]
 
@@ -77,31 +81,50 @@ def _run(cmd: list[str]) -> None:
         sys.stderr.write(proc.stderr)
 
 
+# fp32 arithmetic stays scalar in the sequence-mixing kernels: no packed two-lane fp32 instructions (a device-pass flag;
+# the host pass says it does not know the feature, which is harmless)
+MIX_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
 def _compile(src: Path, force: bool) -> Path:
     obj = OBJ / (src.name + ".o")
     headers = list(CSRC.glob("*.h")) + list(INCLUDE.glob("*.h"))
     if force or _stale(obj, [src] + headers):
-        _run([HIPCC, *COMMON_FLAGS, "-x", "hip", "-c", str(src), "-o", str(obj)])
+        extra = MIX_FLAGS if src.name in MIX_SOURCES else []
+        _run([HIPCC, *COMMON_FLAGS, *extra, "-x", "hip", "-c", str(src), "-o", str(obj)])
     return obj
 
 
-def build_all(force: bool = False, verbose: bool = True) -> dict[str, Path]:
+def build_all(force: bool = False, verbose: bool = True, only=None) -> dict[str, Path]:
+    """Build the shared objects named in `only` (default: all of "hip", "mix", "comm", "gemm")."""
+    want = set(only) if only else {"hip", "mix", "comm", "gemm"}
     LIB.mkdir(exist_ok=True)
     OBJ.mkdir(exist_ok=True)
-    hip_srcs = [CSRC / s for s in HIP_SOURCES if (CSRC / s).exists()]
-    comm_srcs = [CSRC / s for s in COMM_SOURCES if (CSRC / s).exists()]
-    gemm_srcs = [CSRC / s for s in GEMM_SOURCES if (CSRC / s).exists()]
+
+    def srcs(key, names):
+        return [CSRC / s for s in names if (CSRC / s).exists()] if key in want else []
+
+    hip_srcs, mix_srcs = srcs("hip", HIP_SOURCES), srcs("mix", MIX_SOURCES)
+    comm_srcs, gemm_srcs = srcs("comm", COMM_SOURCES), srcs("gemm", GEMM_SOURCES)
+    groups = [hip_srcs, mix_srcs, comm_srcs, gemm_srcs]
     with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
-        objs = list(pool.map(lambda s: _compile(s, force), hip_srcs + comm_srcs + gemm_srcs))
-    hip_objs = objs[: len(hip_srcs)]
-    comm_objs = objs[len(hip_srcs): len(hip_srcs) + len(comm_srcs)]
-    gemm_objs = objs[len(hip_srcs) + len(comm_srcs):]
+        objs = list(pool.map(lambda s: _compile(s, force), [s for g in groups for s in g]))
+    cut = [0]
+    for g in groups:
+        cut.append(cut[-1] + len(g))
+    hip_objs, mix_objs, comm_objs, gemm_objs = (objs[cut[i]: cut[i + 1]] for i in range(4))
     out = {}
-    lib_hip = LIB / "libmsgl_hip.so"
-    if force or _stale(lib_hip, hip_objs):
-        # --no-undefined: a kernel whose host-side launch stub went missing must fail HERE, not at dlopen on the GPU box
-        _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-Wl,--no-undefined", *map(str, hip_objs), "-o", str(lib_hip)])
-    out["hip"] = lib_hip
+    # --no-undefined: a kernel whose host-side launch stub went missing must fail HERE, not at dlopen on the GPU box
+    if hip_objs:
+        lib_hip = LIB / "libmsgl_hip.so"
+        if force or _stale(lib_hip, hip_objs):
+            _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-Wl,--no-undefined", *map(str, hip_objs), "-o", str(lib_hip)])
+        out["hip"] = lib_hip
+    if mix_objs:
+        lib_mix = LIB / "libmsgl_mix.so"
+        if force or _stale(lib_mix, mix_objs):
+            _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-Wl,--no-undefined", *map(str, mix_objs), "-o", str(lib_mix)])
+        out["mix"] = lib_mix
     if comm_objs:
         lib_comm = LIB / "libmsgl_comm.so"
         if force or _stale(lib_comm, comm_objs):

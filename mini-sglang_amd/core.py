@@ -56,13 +56,15 @@ class Req:
 
 
 class Batch:
-    __slots__ = ("reqs", "phase", "input_ids", "positions", "out_loc", "padded_reqs", "attn_metadata")
+    __slots__ = ("reqs", "phase", "input_ids", "positions", "out_loc", "padded_reqs", "attn_metadata", "logit_rows")
 
     def __init__(self, reqs: List[Req], phase: str) -> None:
         if phase not in ("prefill", "decode"):
             raise ValueError(phase)
         self.reqs, self.phase = reqs, phase
         self.padded_reqs: List[Req] = reqs
+        # token indices (device, int) whose logits the forward returns instead of one row per request; None = the usual rows
+        self.logit_rows: Optional[torch.Tensor] = None
 
     is_prefill = property(lambda self: self.phase == "prefill")
     is_decode = property(lambda self: self.phase == "decode")

@@ -154,7 +154,8 @@ int get_handle(hipblasLtHandle_t* h, int* dev_out) {
 }
 
 int make_problem(Problem* p, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int dtype) {
-  const hipDataType t = dtype == MSGL_BF16 ? HIP_R_16BF : HIP_R_16F;
+  // fp32 operands run with HIPBLAS_COMPUTE_32F, the library's true 32-bit mode (no reduced-precision matrix format)
+  const hipDataType t = dtype == MSGL_F32 ? HIP_R_32F : dtype == MSGL_BF16 ? HIP_R_16BF : HIP_R_16F;
   GEMM_BLAS(hipblasLtMatmulDescCreate(&p->desc, HIPBLAS_COMPUTE_32F, HIP_R_32F));
   const int32_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
   GEMM_BLAS(hipblasLtMatmulDescSetAttribute(p->desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta)));
@@ -174,7 +175,7 @@ int check_args(const void* out, const void* x, const void* w, int M, int N, int 
   GEMM_REQUIRE(M >= 1 && N >= 1 && K >= 1, "gemm: bad shape %d x %d x %d", M, N, K);
   GEMM_REQUIRE(ldx >= K && ldw >= K && ldo >= N, "gemm: leading dimensions (%lld, %lld, %lld) too small",
                (long long)ldx, (long long)ldw, (long long)ldo);
-  GEMM_REQUIRE(dtype == MSGL_BF16 || dtype == MSGL_FP16, "gemm: unsupported dtype code %d", dtype);
+  GEMM_REQUIRE(dtype == MSGL_BF16 || dtype == MSGL_FP16 || dtype == MSGL_F32, "gemm: unsupported dtype code %d", dtype);
   return MSGL_OK;
 }
 
@@ -271,7 +272,7 @@ int msgl_gemm_tune(void* out, const void* x, const void* const* w_list, int n_w,
   if ((rc = make_problem(base.prob.get(), M, N, K, ldx, ldw, ldo, dtype)) != MSGL_OK) return rc;
   if ((rc = heuristic_plan(h, &base, ws_bytes)) != MSGL_OK) return rc;
 
-  const hipDataType t = dtype == MSGL_BF16 ? HIP_R_16BF : HIP_R_16F;
+  const hipDataType t = dtype == MSGL_F32 ? HIP_R_32F : dtype == MSGL_BF16 ? HIP_R_16BF : HIP_R_16F;
   // max_candidates: 0 = every library solution, n > 1 = the first n of them, -n = the top n of the
   // library's own heuristic ranking (cheap: tens of candidates), 1 = heuristic pick only
   std::vector<hipblasLtMatmulHeuristicResult_t> all;

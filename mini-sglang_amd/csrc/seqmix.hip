@@ -1,0 +1,728 @@
+// Kernels of the hybrid sequence-mixing models (latent attention + linear-recurrence layers + routed experts),
+// gfx950, wave = 64 lanes.  Built into libmsgl_mix.so; C ABI at the end of the file (include/msgl_mix.h).
+//
+// Precision contract: the residual stream, every norm, rotary angles, attention scores and weights, the recurrent
+// state, router scores and expert weights are fp32 in registers and in memory; tensors that feed a matrix product
+// are stored in the model dtype T (bf16 or fp32).  With T = float every kernel here is true 32-bit.
+//
+//   embed_rows_kernel        x32[t] = table[id[t]]  (+ the T copy the first projection reads)
+//   postnorm_kernel          x32 <- rms(alpha * x32 + sum_p g[t,p] * y[t,p]) * (1 + w)   (+ T copy); also the final norm
+//   latent_prep_kernel       latent row: rms-norm(c) | rotate(k_r) -> cache[out_loc];  rotate(q_r) -> q_abs tail
+//   latent_attn_kernel       one shared (c | k_r) key row for all heads, online softmax, output in latent space
+//   lightning_kernel         S <- decay * S + k v^T, o = S^T q per (request, head), state rows indexed by slot
+//   gated_norm_kernel        rms over the concatenated heads * w * sigmoid(g)
+//   route_kernel             fp32 router: softmax, bias-corrected group-limited top-k, normalised weights
+//   moe_sort_kernel          (token, choice) pairs bucketed by expert -> segment offsets + permutation
+//   gemm_nt_kernel           grouped / segmented / gathered C = act(A B^T): per-head latent products, expert layers,
+//                            and every shape the library refuses
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/msgl_mix.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+void set_err(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+#define MIX_REQUIRE(cond, ...) \
+  do {                         \
+    if (!(cond)) {             \
+      set_err(__VA_ARGS__);    \
+      return MSGL_MIX_EINVAL;  \
+    }                          \
+  } while (0)
+#define MIX_LAUNCHED(name)                                                \
+  do {                                                                    \
+    hipError_t e_ = hipGetLastError();                                    \
+    if (e_ != hipSuccess) {                                               \
+      set_err("%s: launch failed: %s", name, hipGetErrorString(e_));      \
+      return MSGL_MIX_ELAUNCH;                                            \
+    }                                                                     \
+  } while (0)
+
+struct bf16_t {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float ld(const float* p) { return *p; }
+__device__ __forceinline__ float ld(const bf16_t* p) { return __uint_as_float((uint32_t)p->bits << 16); }
+__device__ __forceinline__ void st(float* p, float v) { *p = v; }
+__device__ __forceinline__ void st(bf16_t* p, float v) {  // round to nearest even, NaN kept quiet
+  uint32_t u = __float_as_uint(v);
+  if ((u & 0x7fffffffu) > 0x7f800000u) {
+    p->bits = (uint16_t)((u >> 16) | 0x40u);
+    return;
+  }
+  u += 0x7fffu + ((u >> 16) & 1u);
+  p->bits = (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// sum over a 256-thread workgroup, the same value (and the same order of additions) in every thread
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// ------------------------------------------------------------------------------------------------ embedding
+template <typename T>
+__global__ __launch_bounds__(256) void embed_rows_kernel(float* __restrict__ x32, T* __restrict__ h, const T* __restrict__ table,
+                                                         const int* __restrict__ ids, int W) {
+  const int t = blockIdx.x;
+  const T* row = table + (size_t)ids[t] * W;
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const float v = ld(row + i);
+    x32[(size_t)t * W + i] = v;
+    st(h + (size_t)t * W + i, v);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ post-norm
+// One workgroup per token row.  s = alpha * x + sum_p g[p] * y[p] (fp32, p ascending), out = s * rsqrt(mean(s^2) + eps) * (1 + w).
+template <typename T>
+__global__ __launch_bounds__(256) void postnorm_kernel(const float* __restrict__ x_in, float* __restrict__ x_out, T* __restrict__ h_out,
+                                                       const T* __restrict__ y, int parts, const float* __restrict__ gate,
+                                                       const T* __restrict__ w, float alpha, float eps, int W) {
+  extern __shared__ float srow[];  // W floats + 4
+  float* red = srow + W;
+  const int t = blockIdx.x;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += 256) {
+    float s = alpha * x_in[(size_t)t * W + i];
+    for (int p = 0; p < parts; ++p) {
+      const float yv = ld(y + ((size_t)t * parts + p) * W + i);
+      s = gate ? fmaf(gate[(size_t)t * parts + p], yv, s) : s + yv;
+    }
+    srow[i] = s;
+    ss += s * s;
+  }
+  const float tot = block_sum256(ss, red);
+  const float inv = 1.0f / sqrtf(tot / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const float v = srow[i] * inv * (1.0f + ld(w + i));
+    if (x_out) x_out[(size_t)t * W + i] = v;
+    if (h_out) st(h_out + (size_t)t * W + i, v);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ latent prep
+// One workgroup per token.  proj row = [ q: H x (d + r) | (has_kv) latent R | shared rotated key part r ].
+// cos_sin row p = [cos(p f_i) * amp, i < rd/2 | sin(p f_i) * amp]; the first rd entries of a rotated part turn, the rest pass.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_prep_kernel(const T* __restrict__ proj, int64_t ld_proj, float* __restrict__ q_abs,
+                                                          T* __restrict__ cache, const int* __restrict__ out_loc,
+                                                          const int* __restrict__ positions, const float* __restrict__ cos_sin,
+                                                          const T* __restrict__ c_norm_w, float eps, int H, int d, int r, int rd, int R,
+                                                          int has_kv) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const T* row = proj + (size_t)t * ld_proj;
+  const float* cs = cos_sin + (size_t)positions[t] * rd;
+  const int half = rd >> 1;
+  const int dk = R + r;
+  // rotated query parts -> fp32 tail of the absorbed query rows
+  for (int i = threadIdx.x; i < H * r; i += 256) {
+    const int hh = i / r, j = i - hh * r;
+    const T* qr = row + (size_t)hh * (d + r) + d;
+    float v = ld(qr + j);
+    if (j < rd) {
+      const int pidx = j < half ? j : j - half;
+      const float c = cs[pidx], s = cs[half + pidx];
+      const float u0 = ld(qr + pidx), v0 = ld(qr + pidx + half);
+      v = j < half ? u0 * c - v0 * s : v0 * c + u0 * s;
+    }
+    q_abs[((size_t)t * H + hh) * dk + R + j] = v;
+  }
+  if (!has_kv) return;
+  const T* kv = row + (size_t)H * (d + r);
+  T* dst = cache + (size_t)out_loc[t] * dk;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < R; i += 256) {
+    const float v = ld(kv + i);
+    ss += v * v;
+  }
+  const float inv = 1.0f / sqrtf(block_sum256(ss, red) / (float)R + eps);
+  for (int i = threadIdx.x; i < R; i += 256) st(dst + i, ld(kv + i) * inv * ld(c_norm_w + i));
+  for (int j = threadIdx.x; j < r; j += 256) {
+    float v = ld(kv + R + j);
+    if (j < rd) {
+      const int pidx = j < half ? j : j - half;
+      const float c = cs[pidx], s = cs[half + pidx];
+      const float u0 = ld(kv + R + pidx), v0 = ld(kv + R + pidx + half);
+      v = j < half ? u0 * c - v0 * s : v0 * c + u0 * s;
+    }
+    st(dst + R + j, v);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ latent attention
+// Query rows are (token, head) pairs; all heads read the same key row (latent R | rotated r) and the same value row
+// (the latent).  A workgroup = 16 query rows (QT tokens of one request x HB heads) x 16 lanes; keys in tiles of KT through
+// LDS as fp32; online softmax per row in fp32; output = softmax-weighted latent, fp32.
+constexpr int kAttnRows = 16;
+constexpr int kAttnMaxC = 32;  // value columns per lane: dv <= 512
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_attn_kernel(float* __restrict__ out, const float* __restrict__ q_abs,
+                                                          const T* __restrict__ cache, const int* __restrict__ table,
+                                                          int64_t table_stride, const int* __restrict__ req_rows,
+                                                          const int* __restrict__ seq_lens, const int* __restrict__ cu_q, int B,
+                                                          int H, int dk, int dv, float scale, int QT, int HB, int KT) {
+  extern __shared__ float lds[];
+  const int qs = dk + 1;
+  float* sq = lds;                       // [16][dk + 1]
+  float* sk = sq + kAttnRows * qs;       // [KT][dk + 1]
+  float* sp = sk + KT * qs;              // [16][KT]
+  __shared__ int s_req, s_tok0;
+  if (threadIdx.x == 0) {
+    int g = blockIdx.x, b = 0, found = -1, tok0 = 0;
+    for (; b < B; ++b) {
+      const int n = cu_q[b + 1] - cu_q[b];
+      const int groups = (n + QT - 1) / QT;
+      if (g < groups) {
+        found = b;
+        tok0 = g * QT;
+        break;
+      }
+      g -= groups;
+    }
+    s_req = found;
+    s_tok0 = tok0;
+  }
+  __syncthreads();
+  const int b = s_req;
+  if (b < 0) return;
+  const int q_len = cu_q[b + 1] - cu_q[b];
+  const int start = seq_lens[b] - q_len;  // position of the request's first new token
+  const int h0 = blockIdx.y * HB;
+  const int r = threadIdx.x >> 4, l = threadIdx.x & 15;
+  const int tl = s_tok0 + r / HB, hh = h0 + r % HB;
+  const bool valid = r < QT * HB && tl < q_len && hh < H;
+  const int tok = cu_q[b] + (valid ? tl : s_tok0);
+  const int head = valid ? hh : h0;
+  const int limit = start + (valid ? tl : s_tok0);  // last visible key
+  const int last_tok = min(s_tok0 + QT, q_len) - 1;
+  const int n_keys = start + last_tok + 1;
+  for (int i = l; i < dk; i += 16) sq[r * qs + i] = q_abs[((size_t)tok * H + head) * dk + i];
+  const int* trow = table + (size_t)req_rows[b] * table_stride;
+  float m = -INFINITY, lsum = 0.f;
+  float o[kAttnMaxC];
+#pragma unroll
+  for (int i = 0; i < kAttnMaxC; ++i) o[i] = 0.f;
+  for (int j0 = 0; j0 < n_keys; j0 += KT) {
+    __syncthreads();
+    const int nk = min(KT, n_keys - j0);
+    for (int e = threadIdx.x; e < nk * dk; e += 256) {
+      const int j = e / dk, i = e - j * dk;
+      sk[j * qs + i] = ld(cache + (size_t)trow[j0 + j] * dk + i);
+    }
+    __syncthreads();
+    float tile_max = -INFINITY;
+    for (int j = l; j < KT; j += 16) {
+      float s = -INFINITY;
+      if (j < nk && j0 + j <= limit) {
+        float acc = 0.f;
+        const float* qp = sq + r * qs;
+        const float* kp = sk + j * qs;
+        for (int i = 0; i < dk; ++i) acc = fmaf(qp[i], kp[i], acc);
+        s = acc * scale;
+      }
+      sp[r * KT + j] = s;
+      tile_max = fmaxf(tile_max, s);
+    }
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) tile_max = fmaxf(tile_max, __shfl_xor(tile_max, off, 64));
+    const float m_new = fmaxf(m, tile_max);
+    float corr = 1.f, psum = 0.f;
+    if (m_new > -INFINITY) {
+      corr = expf(m - m_new);
+      for (int j = l; j < KT; j += 16) {
+        const float p = expf(sp[r * KT + j] - m_new);
+        sp[r * KT + j] = p;
+        psum += p;
+      }
+    } else {
+      for (int j = l; j < KT; j += 16) sp[r * KT + j] = 0.f;
+    }
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) psum += __shfl_xor(psum, off, 64);
+    lsum = lsum * corr + psum;
+    m = m_new;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kAttnMaxC; ++i) {
+      const int c = l + 16 * i;
+      if (c < dv) {
+        float acc = o[i] * corr;
+        for (int j = 0; j < nk; ++j) acc = fmaf(sp[r * KT + j], sk[j * qs + c], acc);
+        o[i] = acc;
+      }
+    }
+  }
+  if (!valid) return;
+  const float inv = 1.0f / lsum;
+#pragma unroll
+  for (int i = 0; i < kAttnMaxC; ++i) {
+    const int c = l + 16 * i;
+    if (c < dv) out[((size_t)tok * H + head) * dv + c] = o[i] * inv;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ lightning recurrence
+// Workgroup = one (head, request).  Thread (column v, slice s) keeps rows s, s + NS, ... of column v of the d x dv state in
+// registers.  Tokens go through in batches of kLtTok: q, k, v rows staged in LDS (SiLU applied in fp32), every thread walks
+// the batch sequentially (S <- decay S + k v^T, partial o = sum over its rows of S q), the NS partials of a column are
+// added in slice order.  A request that starts at position 0 starts from a zero state; the state row is the request's slot.
+constexpr int kLtTok = 16;
+constexpr int kLtMaxRows = 64;
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+
+template <typename T>
+__global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out, const T* __restrict__ qkv, int64_t ld_qkv,
+                                                        float* __restrict__ state, const float* __restrict__ decay,
+                                                        const int* __restrict__ cu_q, const int* __restrict__ seq_lens,
+                                                        const int* __restrict__ slots, int H, int d, int dv, int NS) {
+  extern __shared__ float lds[];
+  float* sq = lds;                    // [kLtTok][d]
+  float* skk = sq + kLtTok * d;       // [kLtTok][d]
+  float* sv = skk + kLtTok * d;       // [kLtTok][dv]
+  float* part = sv + kLtTok * dv;     // [kLtTok][NS][dv]
+  const int hh = blockIdx.x, b = blockIdx.y;
+  const int t0 = cu_q[b], n = cu_q[b + 1] - t0;
+  if (n <= 0) return;
+  const bool fresh = seq_lens[b] - n == 0;
+  const int v = threadIdx.x % dv, s = threadIdx.x / dv;
+  const bool active = s < NS;
+  float* S = state + ((size_t)slots[b] * H + hh) * d * dv;
+  const float dec = decay[hh];
+  float reg[kLtMaxRows];
+#pragma unroll
+  for (int i = 0; i < kLtMaxRows; ++i) {
+    const int row = s + i * NS;
+    reg[i] = (active && row < d && !fresh) ? S[(size_t)row * dv + v] : 0.f;
+  }
+  const int64_t qo = (int64_t)hh * d, ko = (int64_t)H * d + (int64_t)hh * d, vo = 2 * (int64_t)H * d + (int64_t)hh * dv;
+  for (int c0 = 0; c0 < n; c0 += kLtTok) {
+    const int nt = min(kLtTok, n - c0);
+    __syncthreads();
+    for (int e = threadIdx.x; e < nt * d; e += 256) {
+      const int tt = e / d, i = e - tt * d;
+      const T* row = qkv + (size_t)(t0 + c0 + tt) * ld_qkv;
+      sq[tt * d + i] = silu_f(ld(row + qo + i));
+      skk[tt * d + i] = silu_f(ld(row + ko + i));
+    }
+    for (int e = threadIdx.x; e < nt * dv; e += 256) {
+      const int tt = e / dv, i = e - tt * dv;
+      sv[tt * dv + i] = silu_f(ld(qkv + (size_t)(t0 + c0 + tt) * ld_qkv + vo + i));
+    }
+    __syncthreads();
+    if (active) {
+      for (int tt = 0; tt < nt; ++tt) {
+        const float vv = sv[tt * dv + v];
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < kLtMaxRows; ++i) {
+          const int row = s + i * NS;
+          if (row < d) {
+            reg[i] = fmaf(dec, reg[i], skk[tt * d + row] * vv);
+            acc = fmaf(reg[i], sq[tt * d + row], acc);
+          }
+        }
+        part[(tt * NS + s) * dv + v] = acc;
+      }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < nt * dv; e += 256) {
+      const int tt = e / dv, i = e - tt * dv;
+      float acc = 0.f;
+      for (int k = 0; k < NS; ++k) acc += part[(tt * NS + k) * dv + i];
+      out[(size_t)(t0 + c0 + tt) * ((size_t)H * dv) + (size_t)hh * dv + i] = acc;
+    }
+  }
+  if (active) {
+#pragma unroll
+    for (int i = 0; i < kLtMaxRows; ++i) {
+      const int row = s + i * NS;
+      if (row < d) S[(size_t)row * dv + v] = reg[i];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ gated norm
+template <typename T>
+__global__ __launch_bounds__(256) void gated_norm_kernel(T* __restrict__ out, const float* __restrict__ o, const T* __restrict__ g,
+                                                         int64_t ld_g, const T* __restrict__ w, float eps, int N) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < N; i += 256) {
+    const float v = o[(size_t)t * N + i];
+    ss += v * v;
+  }
+  const float inv = 1.0f / sqrtf(block_sum256(ss, red) / (float)N + eps);
+  for (int i = threadIdx.x; i < N; i += 256) {
+    const float gate = 1.0f / (1.0f + expf(-ld(g + (size_t)t * ld_g + i)));
+    st(out + (size_t)t * N + i, o[(size_t)t * N + i] * inv * ld(w + i) * gate);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ router
+// One wave per token.  z = W_r h (fp32), s = softmax(z); choice = s + bias; experts outside the `keep` best groups (a group's
+// score = its largest choice) are out; the `top` largest choices win (ties: lowest index); weight = s / (sum of chosen s + 1e-20).
+template <typename T>
+__global__ __launch_bounds__(64) void route_kernel(int* __restrict__ ids, float* __restrict__ wts, const T* __restrict__ h,
+                                                   const T* __restrict__ router, const T* __restrict__ bias, int E, int top, int G,
+                                                   int keep, int W) {
+  extern __shared__ float lds[];
+  float* s = lds;           // [E] softmax scores
+  float* c = s + E;         // [E] choice scores
+  float* gs = c + E;        // [G]
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const T* x = h + (size_t)t * W;
+  for (int e = 0; e < E; ++e) {
+    float acc = 0.f;
+    for (int i = lane; i < W; i += 64) acc = fmaf(ld(x + i), ld(router + (size_t)e * W + i), acc);
+    acc = wave_sum(acc);
+    if (lane == 0) s[e] = acc;
+  }
+  __syncthreads();
+  if (lane == 0) {
+    float mx = -INFINITY;
+    for (int e = 0; e < E; ++e) mx = fmaxf(mx, s[e]);
+    float sum = 0.f;
+    for (int e = 0; e < E; ++e) {
+      s[e] = expf(s[e] - mx);
+      sum += s[e];
+    }
+    for (int e = 0; e < E; ++e) {
+      s[e] /= sum;
+      c[e] = s[e] + (bias ? ld(bias + e) : 0.f);
+    }
+    const int per = E / G;
+    if (keep < G) {
+      for (int g = 0; g < G; ++g) {
+        float b = -INFINITY;
+        for (int e = g * per; e < (g + 1) * per; ++e) b = fmaxf(b, c[e]);
+        gs[g] = b;
+      }
+      // a group stays if fewer than `keep` groups beat it (ties: the lower index wins)
+      for (int g = 0; g < G; ++g) {
+        int better = 0;
+        for (int o2 = 0; o2 < G; ++o2) better += (gs[o2] > gs[g]) || (gs[o2] == gs[g] && o2 < g);
+        if (better >= keep)
+          for (int e = g * per; e < (g + 1) * per; ++e) c[e] = -INFINITY;
+      }
+    }
+    float tot = 0.f;
+    for (int k = 0; k < top; ++k) {
+      int best = -1;
+      float bv = -INFINITY;
+      for (int e = 0; e < E; ++e)
+        if (c[e] > bv) {
+          best = e;
+          bv = c[e];
+        }
+      if (best < 0) best = 0;  // unreachable: the host checks top <= keep * (E / G) and choice scores are finite
+      ids[(size_t)t * top + k] = best;
+      wts[(size_t)t * top + k] = s[best];
+      tot += s[best];
+      c[best] = -INFINITY;
+    }
+    for (int k = 0; k < top; ++k) wts[(size_t)t * top + k] /= (tot + 1e-20f);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ expert bucketing
+// One workgroup.  seg[e] .. seg[e + 1] = the sorted positions of expert e; perm[position] = flat (token * top + choice).
+// Positions inside a segment follow the flat index (stable), so the layout does not depend on scheduling.
+__global__ __launch_bounds__(256) void moe_sort_kernel(int* __restrict__ seg, int* __restrict__ perm, const int* __restrict__ ids, int n,
+                                                       int E) {
+  extern __shared__ int li[];  // [E + 1]
+  for (int e = threadIdx.x; e <= E; e += 256) li[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += 256) atomicAdd(&li[ids[i] + 1], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int e = 0; e < E; ++e) li[e + 1] += li[e];
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e <= E; e += 256) seg[e] = li[e];
+  // stable placement: thread e walks the flat list for its expert
+  for (int e = threadIdx.x; e < E; e += 256) {
+    int p = li[e];
+    for (int i = 0; i < n; ++i)
+      if (ids[i] == e) perm[p++] = i;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ grouped GEMM
+// C[g][m][n] = act(sum_k A[g][m][k] * B[g][n][k]), fp32 accumulation in a fixed k order.
+//   groups: A, B, C advance by a_gs, b_gs, c_gs elements per group (heads of one projection, experts);
+//   seg != null: group g owns rows seg[g] .. seg[g + 1] of the row space (expert segments), M is an upper bound;
+//   a_rows / c_rows != null: the row space is indirect (row m of A is a_rows[m] / a_div, row m of C is c_rows[m]).
+// 64 x 64 tile, 256 threads, 4 x 4 outputs per thread, k in steps of 16 through LDS.
+constexpr int kTile = 64, kStepK = 16;
+
+template <typename TA, typename TB, typename TC>
+__global__ __launch_bounds__(256) void gemm_nt_kernel(TC* __restrict__ C, const TA* __restrict__ A, const TB* __restrict__ Bm, int M, int N,
+                                                      int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t a_gs, int64_t b_gs,
+                                                      int64_t c_gs, const int* __restrict__ seg, const int* __restrict__ a_rows, int a_div,
+                                                      const int* __restrict__ c_rows, int act) {
+  __shared__ float sa[kStepK][kTile + 1];
+  __shared__ float sb[kStepK][kTile + 1];
+  const int g = blockIdx.z;
+  int row0 = 0, rows = M;
+  if (seg) {
+    row0 = seg[g];
+    rows = seg[g + 1] - row0;
+  }
+  const int m0 = blockIdx.y * kTile, n0 = blockIdx.x * kTile;
+  if (m0 >= rows) return;
+  const TA* Ag = A + (seg ? 0 : g * a_gs);
+  const TB* Bg = Bm + g * b_gs;
+  TC* Cg = C + (seg ? 0 : g * c_gs);
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  // loader mapping: thread -> (row of the tile = tid / 4, four consecutive k = (tid % 4) * 4)
+  const int lr = threadIdx.x >> 2, lk = (threadIdx.x & 3) * 4;
+  int64_t a_off = -1;
+  if (m0 + lr < rows) {
+    const int m = row0 + m0 + lr;
+    a_off = (int64_t)(a_rows ? a_rows[m] / a_div : m) * lda;
+  }
+  const int64_t b_off = n0 + lr < N ? (int64_t)(n0 + lr) * ldb : -1;
+  for (int k0 = 0; k0 < K; k0 += kStepK) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k = k0 + lk + u;
+      sa[lk + u][lr] = (a_off >= 0 && k < K) ? ld(Ag + a_off + k) : 0.f;
+      sb[lk + u][lr] = (b_off >= 0 && k < K) ? ld(Bg + b_off + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < kStepK; ++kk) {
+      float av[4], bv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = sa[kk][ty + 16 * i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bv[j] = sb[kk][tx + 16 * j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int ml = m0 + ty + 16 * i;
+    if (ml >= rows) continue;
+    const int m = row0 + ml;
+    const int64_t c_off = (int64_t)(c_rows ? c_rows[m] : m) * ldc;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx + 16 * j;
+      if (n >= N) continue;
+      float v = acc[i][j];
+      if (act == MSGL_MIX_ACT_RELU2) {
+        v = fmaxf(v, 0.f);
+        v = v * v;
+      }
+      st(Cg + c_off + n, v);
+    }
+  }
+}
+
+template <typename T>
+const T* cp(const void* p) {
+  return static_cast<const T*>(p);
+}
+template <typename T>
+T* mp(void* p) {
+  return static_cast<T*>(p);
+}
+
+bool dtype_ok(int dt) { return dt == MSGL_MIX_BF16 || dt == MSGL_MIX_F32; }
+
+int ensure_lds(const void* fn, size_t bytes) {
+  if (bytes <= 64 * 1024) return 0;
+  if (bytes > 160 * 1024) return -1;
+  return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) == hipSuccess ? 0 : -1;
+}
+
+}  // namespace
+
+#define DISPATCH_T(dt, ...)          \
+  if ((dt) == MSGL_MIX_BF16) {       \
+    using T = bf16_t;                \
+    __VA_ARGS__                      \
+  } else {                           \
+    using T = float;                 \
+    __VA_ARGS__                      \
+  }
+
+extern "C" {
+
+const char* msgl_mix_last_error(void) { return g_err; }
+int msgl_mix_abi_version(void) { return MSGL_MIX_ABI_VERSION; }
+
+int msgl_mix_embed(float* x32, void* h, const void* table, const int* ids, int tokens, int W, int dtype, void* stream) {
+  MIX_REQUIRE(x32 && h && table && ids && tokens >= 0 && W >= 1 && dtype_ok(dtype), "embed: bad arguments");
+  if (tokens == 0) return MSGL_MIX_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, hipLaunchKernelGGL(embed_rows_kernel<T>, dim3(tokens), dim3(256), 0, s, x32, mp<T>(h), cp<T>(table), ids, W);)
+  MIX_LAUNCHED("embed");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_postnorm(const float* x_in, float* x_out, void* h_out, const void* y, int parts, const float* gate, const void* w,
+                      float alpha, float eps, int rows, int W, int dtype, void* stream) {
+  MIX_REQUIRE(x_in && w && (x_out || h_out) && rows >= 0 && W >= 1 && dtype_ok(dtype), "postnorm: bad arguments");
+  MIX_REQUIRE((parts == 0) == (y == nullptr) && parts >= 0, "postnorm: parts = %d does not match y", parts);
+  if (rows == 0) return MSGL_MIX_OK;
+  const size_t lds = (size_t)(W + 4) * sizeof(float);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)postnorm_kernel<T>, lds) == 0, "postnorm: row of %d does not fit LDS", W);
+             hipLaunchKernelGGL(postnorm_kernel<T>, dim3(rows), dim3(256), lds, s, x_in, x_out, mp<T>(h_out), cp<T>(y), parts, gate,
+                                cp<T>(w), alpha, eps, W);)
+  MIX_LAUNCHED("postnorm");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_latent_prep(const void* proj, int64_t ld_proj, float* q_abs, void* cache, const int* out_loc, const int* positions,
+                         const float* cos_sin, const void* c_norm_w, float eps, int tokens, int H, int d, int r, int rot_dims, int R,
+                         int has_kv, int dtype, void* stream) {
+  MIX_REQUIRE(proj && q_abs && positions && cos_sin && dtype_ok(dtype), "latent_prep: null pointer / dtype");
+  MIX_REQUIRE(H >= 1 && d >= 0 && r >= 0 && R >= 1 && rot_dims >= 0 && rot_dims <= r && rot_dims % 2 == 0,
+              "latent_prep: bad sizes H %d d %d r %d rot %d R %d", H, d, r, rot_dims, R);
+  MIX_REQUIRE(!has_kv || (cache && out_loc && c_norm_w), "latent_prep: a layer with its own latent needs cache, out_loc and norm weight");
+  MIX_REQUIRE(ld_proj >= (int64_t)H * (d + r) + (has_kv ? R + r : 0), "latent_prep: projection row too short");
+  if (tokens == 0) return MSGL_MIX_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, hipLaunchKernelGGL(latent_prep_kernel<T>, dim3(tokens), dim3(256), 0, s, cp<T>(proj), ld_proj, q_abs, mp<T>(cache),
+                                       out_loc, positions, cos_sin, cp<T>(c_norm_w), eps, H, d, r, rot_dims, R, has_kv);)
+  MIX_LAUNCHED("latent_prep");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, const int* table, int64_t table_stride, const int* req_rows,
+                         const int* seq_lens, const int* cu_q, int batch, int total_q, int H, int dk, int dv, float scale, int dtype,
+                         void* stream) {
+  MIX_REQUIRE(out && q_abs && cache && table && req_rows && seq_lens && cu_q && dtype_ok(dtype), "latent_attn: null pointer / dtype");
+  MIX_REQUIRE(batch >= 1 && total_q >= 0 && H >= 1 && dv >= 1 && dk >= dv, "latent_attn: bad sizes");
+  MIX_REQUIRE(dv <= 16 * kAttnMaxC, "latent_attn: value width %d above %d", dv, 16 * kAttnMaxC);
+  if (total_q == 0) return MSGL_MIX_OK;
+  const int HB = H < kAttnRows ? H : kAttnRows;
+  const int QT = kAttnRows / HB;
+  int KT = 64;
+  auto need = [&](int kt) { return (size_t)((kAttnRows + kt) * (dk + 1) + kAttnRows * kt) * sizeof(float); };
+  while (KT > 8 && need(KT) > 160 * 1024) KT >>= 1;
+  const size_t lds = need(KT);
+  MIX_REQUIRE(lds <= 160 * 1024, "latent_attn: key width %d does not fit LDS", dk);
+  const int groups = (total_q + QT - 1) / QT + batch;  // every request may end with one partial group
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)latent_attn_kernel<T>, lds) == 0, "latent_attn: LDS request refused");
+             hipLaunchKernelGGL(latent_attn_kernel<T>, dim3(groups, (H + HB - 1) / HB), dim3(256), lds, s, out, q_abs, cp<T>(cache), table,
+                                table_stride, req_rows, seq_lens, cu_q, batch, H, dk, dv, scale, QT, HB, KT);)
+  MIX_LAUNCHED("latent_attn");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_lightning(float* out, const void* qkv, int64_t ld_qkv, float* state, const float* decay, const int* cu_q, const int* seq_lens,
+                       const int* slots, int batch, int H, int d, int dv, int dtype, void* stream) {
+  MIX_REQUIRE(out && qkv && state && decay && cu_q && seq_lens && slots && dtype_ok(dtype), "lightning: null pointer / dtype");
+  MIX_REQUIRE(batch >= 1 && H >= 1 && d >= 1 && dv >= 1 && dv <= 256, "lightning: bad sizes (value width %d, at most 256)", dv);
+  MIX_REQUIRE(ld_qkv >= (int64_t)H * (2 * d + dv), "lightning: projection row too short");
+  const int NS = 256 / dv;
+  MIX_REQUIRE((d + NS - 1) / NS <= kLtMaxRows, "lightning: state %d x %d needs more than %d rows per thread", d, dv, kLtMaxRows);
+  const size_t lds = (size_t)(kLtTok * (2 * d + dv) + kLtTok * NS * dv) * sizeof(float);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)lightning_kernel<T>, lds) == 0, "lightning: LDS request refused");
+             hipLaunchKernelGGL(lightning_kernel<T>, dim3(H, batch), dim3(256), lds, s, out, cp<T>(qkv), ld_qkv, state, decay, cu_q,
+                                seq_lens, slots, H, d, dv, NS);)
+  MIX_LAUNCHED("lightning");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_gated_norm(void* out, const float* o, const void* gate, int64_t ld_gate, const void* w, float eps, int rows, int N, int dtype,
+                        void* stream) {
+  MIX_REQUIRE(out && o && gate && w && rows >= 0 && N >= 1 && ld_gate >= N && dtype_ok(dtype), "gated_norm: bad arguments");
+  if (rows == 0) return MSGL_MIX_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, hipLaunchKernelGGL(gated_norm_kernel<T>, dim3(rows), dim3(256), 0, s, mp<T>(out), o, cp<T>(gate), ld_gate, cp<T>(w), eps, N);)
+  MIX_LAUNCHED("gated_norm");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_route(int* ids, float* wts, const void* h, const void* router, const void* bias, int tokens, int W, int E, int top, int G,
+                   int keep, int dtype, void* stream) {
+  MIX_REQUIRE(ids && wts && h && router && dtype_ok(dtype), "route: null pointer / dtype");
+  MIX_REQUIRE(E >= 1 && top >= 1 && top <= E && G >= 1 && E % G == 0 && keep >= 1 && keep <= G && top <= keep * (E / G),
+              "route: bad sizes E %d top %d groups %d keep %d", E, top, G, keep);
+  if (tokens == 0) return MSGL_MIX_OK;
+  const size_t lds = (size_t)(2 * E + G) * sizeof(float);
+  MIX_REQUIRE(lds <= 64 * 1024, "route: too many experts");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, hipLaunchKernelGGL(route_kernel<T>, dim3(tokens), dim3(64), lds, s, ids, wts, cp<T>(h), cp<T>(router), cp<T>(bias), E, top,
+                                       G, keep, W);)
+  MIX_LAUNCHED("route");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_moe_sort(int* seg, int* perm, const int* ids, int n, int E, void* stream) {
+  MIX_REQUIRE(seg && perm && ids && n >= 0 && E >= 1 && E <= 8192, "moe_sort: bad arguments");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(256), (size_t)(E + 1) * sizeof(int), s, seg, perm, ids, n, E);
+  MIX_LAUNCHED("moe_sort");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_gemm_nt(void* C, const void* A, const void* B, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int groups,
+                     int64_t a_gs, int64_t b_gs, int64_t c_gs, const int* seg, const int* a_rows, int a_div, const int* c_rows, int act,
+                     int ta, int tb, int tc, void* stream) {
+  MIX_REQUIRE(C && A && B && M >= 0 && N >= 1 && K >= 1 && groups >= 1 && groups <= 65535, "gemm_nt: bad arguments");
+  MIX_REQUIRE(dtype_ok(ta) && dtype_ok(tb) && dtype_ok(tc), "gemm_nt: dtype codes");
+  MIX_REQUIRE(lda >= K && ldb >= K && a_div >= 1, "gemm_nt: leading dimensions");
+  MIX_REQUIRE(act == MSGL_MIX_ACT_NONE || act == MSGL_MIX_ACT_RELU2, "gemm_nt: activation code %d", act);
+  if (M == 0) return MSGL_MIX_OK;
+  const int row_tiles = (M + kTile - 1) / kTile;
+  MIX_REQUIRE(row_tiles <= 65535, "gemm_nt: too many rows");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((N + kTile - 1) / kTile, row_tiles, groups);
+#define GEMM_CASE(CA, CB, CC, TA, TB, TC)                                                                                            \
+  if (ta == CA && tb == CB && tc == CC) {                                                                                            \
+    hipLaunchKernelGGL((gemm_nt_kernel<TA, TB, TC>), grid, dim3(256), 0, s, mp<TC>(C), cp<TA>(A), cp<TB>(B), M, N, K, lda, ldb, ldc, \
+                       a_gs, b_gs, c_gs, seg, a_rows, a_div, c_rows, act);                                                           \
+    MIX_LAUNCHED("gemm_nt");                                                                                                         \
+    return MSGL_MIX_OK;                                                                                                              \
+  }
+  GEMM_CASE(MSGL_MIX_BF16, MSGL_MIX_BF16, MSGL_MIX_BF16, bf16_t, bf16_t, bf16_t)
+  GEMM_CASE(MSGL_MIX_BF16, MSGL_MIX_BF16, MSGL_MIX_F32, bf16_t, bf16_t, float)
+  GEMM_CASE(MSGL_MIX_F32, MSGL_MIX_BF16, MSGL_MIX_BF16, float, bf16_t, bf16_t)
+  GEMM_CASE(MSGL_MIX_F32, MSGL_MIX_F32, MSGL_MIX_F32, float, float, float)
+#undef GEMM_CASE
+  set_err("gemm_nt: no kernel for dtype codes (%d, %d, %d)", ta, tb, tc);
+  return MSGL_MIX_EINVAL;
+}
+
+}  // extern "C"

@@ -18,9 +18,10 @@ import torch
 
 from . import flashinfer_compat as fi
 from . import ops
-from .attention import HipAttnBackend
+from .attention import HipAttnBackend, MixAttnBackend
 from .core import Batch, Context, Req, SamplingParams, set_global_ctx
-from .kvcache import create_kvcache_pool, heads_per_rank
+from .hybrid import HybridConfig, HybridDecoder
+from .kvcache import HybridCache, create_kvcache_pool, heads_per_rank
 from .model import Communicator, DenseDecoder, ModelConfig
 
 
@@ -103,7 +104,7 @@ BatchSamplingArgs = SamplingPlan  # the reference's name for the record
 @dataclass
 class EngineConfig:
     """Fields of P/engine/config.py:16-55 that reach the hot path."""
-    model: ModelConfig
+    model: Any  # ModelConfig (dense families) or HybridConfig
     dtype: torch.dtype = torch.bfloat16
     tp_rank: int = 0
     tp_size: int = 1
@@ -143,10 +144,14 @@ def _align_up_32(n: int) -> int:
 def determine_num_pages(free_before: int, free_after: int, cfg: EngineConfig) -> int:
     """P/engine/engine.py:148-168: (memory_ratio * free_before - model_bytes) // bytes_per_page."""
     m = cfg.model
-    cache_per_page = (2 * m.head_dim * heads_per_rank(m.num_kv_heads, cfg.tp_size, replicate=True) * cfg.page_size
-                      * torch.empty((), dtype=cfg.dtype).element_size() * m.num_layers)
     if cfg.num_page_override is not None:
         return cfg.num_page_override
+    if isinstance(m, HybridConfig):  # one shared latent row per token and caching layer; the recurrent states are a fixed cost
+        cache_per_page = max(HybridCache.bytes_per_page(m.layers, cfg.page_size, cfg.dtype), 1)
+        free_after -= HybridCache.state_bytes(m.layers, cfg.max_running_req + 1)
+    else:
+        cache_per_page = (2 * m.head_dim * heads_per_rank(m.num_kv_heads, cfg.tp_size, replicate=True) * cfg.page_size
+                          * torch.empty((), dtype=cfg.dtype).element_size() * m.num_layers)
     model_memory = free_before - free_after
     available = int(cfg.memory_ratio * free_before) - model_memory
     num_pages = available // cache_per_page
@@ -264,21 +269,30 @@ class Engine:
         # two collectives of ONE communicator must never be in flight at once (shared flags / sequence counters; RCCL is
         # not safe across two streams either): without a second communicator the token halves run serially
         overlap = cfg.comm_overlap and not (cfg.tp_size > 1 and cfg.comm_split_tokens > 0 and cfg.comm_side is None)
-        self.model = DenseDecoder(cfg.model, dtype=cfg.dtype, device=self.device, tp_rank=cfg.tp_rank,
-                                  tp_size=cfg.tp_size, seed=cfg.seed, comm=comm, fused=cfg.fused_qkv_path,
-                                  comm_split_tokens=cfg.comm_split_tokens, comm_overlap=overlap)
+        hybrid = isinstance(cfg.model, HybridConfig)
+        if hybrid:  # its rotary tables end at the engine's sequence limit: the design states no maximum position
+            self.model = HybridDecoder(cfg.model, dtype=cfg.dtype, device=self.device, tp_rank=cfg.tp_rank, tp_size=cfg.tp_size,
+                                       seed=cfg.seed, max_position=_align_up_32(
+                                           cfg.max_seq_len if cfg.num_page_override is None
+                                           else min(cfg.max_seq_len, cfg.num_page_override * cfg.page_size)) + 1)
+        else:
+            self.model = DenseDecoder(cfg.model, dtype=cfg.dtype, device=self.device, tp_rank=cfg.tp_rank,
+                                      tp_size=cfg.tp_size, seed=cfg.seed, comm=comm, fused=cfg.fused_qkv_path,
+                                      comm_split_tokens=cfg.comm_split_tokens, comm_overlap=overlap)
         torch.cuda.synchronize(self.device)
         free_after = self._agreed_free_memory(torch.cuda.mem_get_info(self.device)[0])
 
         self.num_pages = determine_num_pages(free_before, free_after, cfg)
         num_tokens = self.num_pages * cfg.page_size
         self.ctx.kv_cache = self.kv_cache = create_kvcache_pool(
-            cfg.model, self.num_pages + 1, cfg.page_size, cfg.dtype, self.device, tp_size=cfg.tp_size)  # +1 dummy
+            cfg.model, self.num_pages + 1, cfg.page_size, cfg.dtype, self.device, tp_size=cfg.tp_size,
+            state_rows=cfg.max_running_req + 1)  # +1 page / +1 state row: the dummy request's
         self.max_seq_len = min(cfg.max_seq_len, num_tokens)
         self.aligned_max_seq_len = _align_up_32(self.max_seq_len)
         self.ctx.page_table = self.page_table = torch.zeros(
             (cfg.max_running_req + 1, self.aligned_max_seq_len), dtype=torch.int32, device=self.device)
-        self.ctx.attn_backend = self.attn_backend = HipAttnBackend(cfg.model, self.ctx, tp_size=cfg.tp_size)
+        self.ctx.attn_backend = self.attn_backend = (MixAttnBackend if hybrid else HipAttnBackend)(
+            cfg.model, self.ctx, tp_size=cfg.tp_size)
         self.sampler = Sampler(self.device, cfg.model.vocab_size)
         self.dummy_req = Req(input_ids=torch.tensor([0], dtype=torch.int32), table_idx=cfg.max_running_req,
                              cached_len=0, output_len=1, uid=-1)
@@ -290,7 +304,7 @@ class Engine:
                                                  prefill_tokens=[cfg.prefill_tokens] if cfg.prefill_tokens else ())
         self.graph_runner = GraphRunner(self, bs_list)
         self.refine_report: List[dict] = []
-        if cfg.refine_in_graph and cfg.gemm_tune != "off" and bs_list and cfg.tp_size == 1 and \
+        if cfg.refine_in_graph and cfg.gemm_tune != "off" and bs_list and cfg.tp_size == 1 and not hybrid and \
                 os.environ.get("MSGL_DISABLE_REFINE") != "1":
             self.refine_report = self.refine_plans_in_graph(max(bs_list))
         if cfg.tp_size > 1 and cfg.tp_cpu_group is not None:
@@ -314,6 +328,19 @@ class Engine:
             row_len=self.aligned_max_seq_len, device=self.device, Req=Req, Batch=Batch,
             prepare_metadata=self.attn_backend.prepare_metadata, capture=lambda: gr.capture(bs), replay=gr.replay,
             forward_ctx=self.ctx.forward_batch)
+
+    def forward_logits(self, batch: Batch) -> torch.Tensor:
+        """The forward of `forward_batch` without the draw: logits at `batch.logit_rows` (or the model's usual rows), and the
+        same host bookkeeping -- everything on the device counts as cached afterwards.  For callers that force the tokens
+        themselves (a recorded trace, scoring)."""
+        with self.ctx.forward_batch(batch):
+            if batch.logit_rows is None and self.graph_runner.can_use_cuda_graph(batch):
+                logits = self.graph_runner.replay(batch)
+            else:
+                logits = self.model.forward(self.ctx, batch)
+        for req in batch.reqs:
+            req.cached_len = req.device_len
+        return logits
 
     def _agreed_free_memory(self, free: int) -> int:
         """Every TP rank must derive the same num_pages / max_seq_len / page-table width (the schedulers are

@@ -76,14 +76,31 @@ def _cos_sin_cache(rotary_dim: int, max_position: int, base: float,
         beta_fast = rope_scaling.get("beta_fast", 32.0)
         beta_slow = rope_scaling.get("beta_slow", 1.0)
         orig = rope_scaling["original_max_position_embeddings"]
+        # variants of the ramp that other designs fix differently: where its upper end is capped, the smallest span it
+        # divides by, and an amplitude on cos and sin (the defaults are the reference's)
+        hi_cap = rope_scaling.get("hi_cap", rotary_dim // 2 - 1)
+        min_span = rope_scaling.get("min_span", 1)
+        amplitude = float(rope_scaling.get("amplitude", 1.0))
 
         def corr_dim(rotations: float) -> float:
             return rotary_dim * math.log(orig / (rotations * 2 * math.pi)) / (2 * math.log(base))
 
         lo = max(math.floor(corr_dim(beta_fast)), 0)
-        hi = min(math.ceil(corr_dim(beta_slow)), rotary_dim // 2 - 1)
-        ramp = torch.clamp((torch.arange(rotary_dim // 2, dtype=torch.float32) - lo) / max(hi - lo, 1), 0, 1)
+        hi = min(math.ceil(corr_dim(beta_slow)), hi_cap)
+        if rope_scaling.get("float64_table"):
+            # angles from float64 frequencies, rounded once: for models whose whole rotary path is held to fp32 accuracy
+            i64 = torch.arange(rotary_dim // 2, dtype=torch.float64)
+            f64 = base ** (-2.0 * i64 / rotary_dim)
+            ramp = torch.clamp((i64 - lo) / max(hi - lo, min_span), 0, 1)
+            f64 = (f64 / factor) * ramp + f64 * (1 - ramp)
+            ang = torch.arange(max_position, dtype=torch.float64)[:, None] * f64[None, :]
+            return torch.cat((ang.cos() * amplitude, ang.sin() * amplitude), dim=-1).to(torch.float32)
+        ramp = torch.clamp((torch.arange(rotary_dim // 2, dtype=torch.float32) - lo) / max(hi - lo, min_span), 0, 1)
         inv_freq = (inv_freq / factor) * ramp + inv_freq * (1 - ramp)
+        if amplitude != 1.0:
+            t = torch.arange(max_position, dtype=torch.float)
+            freqs = torch.einsum("i,j -> ij", t, inv_freq)
+            return torch.cat((freqs.cos() * amplitude, freqs.sin() * amplitude), dim=-1)
     elif kind not in (None, "default"):
         raise ValueError(f"Unsupported rope_scaling = {rope_scaling}")
     t = torch.arange(max_position, dtype=torch.float)

@@ -76,8 +76,70 @@ class MHAKVCache:
 
 
 def create_kvcache_pool(model_config, num_pages: int, page_size: int, dtype: torch.dtype, device: torch.device,
-                        tp_size: int = 1) -> MHAKVCache:
-    """P/kvcache/__init__.py:27-44."""
+                        tp_size: int = 1, state_rows: int = 0):
+    """P/kvcache/__init__.py:27-44; a configuration that lists its layers one by one (`layers` of specs) gets the per-layer
+    HybridCache with `state_rows` recurrent-state slots."""
+    if hasattr(model_config, "layers"):
+        return HybridCache(model_config.layers, num_pages, page_size, state_rows, dtype, device)
     return MHAKVCache(num_kv_heads=model_config.num_kv_heads, num_pages=num_pages, page_size=page_size,
                       num_layers=model_config.num_layers, head_dim=model_config.head_dim, device=device,
                       dtype=dtype, tp_size=tp_size)
+
+
+class HybridCache:
+    """Per-layer memory of a model that mixes latent-attention layers with linear-recurrence layers.
+
+    * a latent-attention layer that owns its keys caches ONE row per token, shared by all heads: `latent_rows(layer)` is
+      `[num_pages * page_size, kv_rank + rot_dim]` in the model dtype, indexed by the same token slots of the global page
+      table as the MHA pool (the extra last page is the dummy target of padded rows); a layer that borrows another layer's
+      keys has no rows of its own and is handed the owner's;
+    * a linear-recurrence layer keeps one fp32 state `[heads, dim, vdim]` per running request: `state(layer)` is
+      `[state_rows, heads, dim, vdim]`, indexed by the request's page-table row, so a row that is handed to a new request
+      brings its state slot with it (the kernel starts a request whose first token is at position 0 from zero).
+    Layers may differ in every size, so each gets its own allocation.
+    """
+
+    def __init__(self, layers, num_pages: int, page_size: int, state_rows: int, dtype: torch.dtype, device: torch.device) -> None:
+        self._latent, self._state, self._owner = {}, {}, {}
+        slots = num_pages * page_size
+        for i, spec in enumerate(layers):
+            if spec.kind == "latent_attention":
+                if spec.kv_from is None:
+                    self._latent[i] = torch.zeros((slots, spec.kv_rank + spec.rot_dim), dtype=dtype, device=device)
+                self._owner[i] = i if spec.kv_from is None else spec.kv_from
+            elif spec.kind == "lightning":
+                self._state[i] = torch.zeros((state_rows, spec.heads, spec.dim, spec.vdim), dtype=torch.float32, device=device)
+        for i, j in self._owner.items():
+            if j not in self._latent:
+                raise ValueError(f"layer {i} borrows the keys of layer {j}, which caches none")
+        self._dtype, self._device, self._layers = dtype, device, len(layers)
+
+    def latent_rows(self, layer: int) -> torch.Tensor:
+        return self._latent[self._owner[layer]]
+
+    def owns_latent(self, layer: int) -> bool:
+        return layer in self._latent
+
+    def state(self, layer: int) -> torch.Tensor:
+        return self._state[layer]
+
+    @staticmethod
+    def bytes_per_page(layers, page_size: int, dtype: torch.dtype) -> int:
+        es = torch.empty((), dtype=dtype).element_size()
+        return sum((s.kv_rank + s.rot_dim) * es * page_size for s in layers if s.kind == "latent_attention" and s.kv_from is None)
+
+    @staticmethod
+    def state_bytes(layers, state_rows: int) -> int:
+        return sum(4 * s.heads * s.dim * s.vdim * state_rows for s in layers if s.kind == "lightning")
+
+    @property
+    def device(self) -> torch.device:
+        return self._device
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self._dtype
+
+    @property
+    def num_layers(self) -> int:
+        return self._layers

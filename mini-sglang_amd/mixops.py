@@ -1,0 +1,197 @@
+"""torch-facing wrappers of the sequence-mixing kernels (include/msgl_mix.h, csrc/seqmix.hip).
+
+Same rules as ops.py: device tensors only, no CPU fallback, pointers + sizes + the current stream go straight to
+the C ABI.  `linear` is the projection seam of the hybrid models: the library GEMM (bf16, or fp32 in the library's
+true 32-bit mode) and, for shapes the library has no solution for, the grouped kernel of this file.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib, ops
+from ._lib import check_mix, mix_lib
+
+ACT_NONE, ACT_RELU2 = 0, 1
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return _lib.BF16
+    if t.dtype == torch.float32:
+        return _lib.F32
+    raise TypeError(f"expected a bf16 or fp32 tensor, got {t.dtype}")
+
+
+def _dev(*ts: Optional[torch.Tensor]) -> None:
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("mini_sglang_amd mixops run on the HIP device only (got a CPU tensor)")
+
+
+def _i32(t: torch.Tensor) -> torch.Tensor:
+    assert t.dtype == torch.int32 and t.is_contiguous(), (t.dtype, t.stride())
+    return t
+
+
+def _p(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def embed(table: torch.Tensor, ids: torch.Tensor):
+    """-> (fp32 rows, the same rows in the table's dtype)."""
+    _dev(table, ids)
+    assert table.dim() == 2 and table.is_contiguous()
+    T, W = ids.shape[0], table.shape[1]
+    x32 = torch.empty((T, W), dtype=torch.float32, device=table.device)
+    h = torch.empty((T, W), dtype=table.dtype, device=table.device)
+    check_mix(mix_lib().msgl_mix_embed(x32.data_ptr(), h.data_ptr(), table.data_ptr(), _i32(ids).data_ptr(), T, W,
+                                       _code(table), _stream()), "embed")
+    return x32, h
+
+
+def postnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, *, y: Optional[torch.Tensor] = None,
+             gate: Optional[torch.Tensor] = None, alpha: float = 1.0, x_out: Optional[torch.Tensor] = None,
+             h_out: Optional[torch.Tensor] = None) -> None:
+    """s = alpha x + sum_p gate[:, p] y[:, p];  out = rms_unit(s) * (1 + weight) -> x_out (fp32) and / or h_out (weight's dtype).
+    y: [rows, W] or [rows, parts, W]."""
+    _dev(x, weight, y, gate, x_out, h_out)
+    rows, W = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous() and weight.shape == (W,) and weight.is_contiguous()
+    parts = 0
+    if y is not None:
+        assert y.is_contiguous() and y.dtype == weight.dtype and y.shape[0] == rows and y.shape[-1] == W
+        parts = 1 if y.dim() == 2 else y.shape[1]
+    if gate is not None:
+        assert gate.dtype == torch.float32 and gate.is_contiguous() and gate.numel() == rows * parts
+    for o, dt in ((x_out, torch.float32), (h_out, weight.dtype)):
+        assert o is None or (o.shape == (rows, W) and o.is_contiguous() and o.dtype == dt)
+    if rows == 0:
+        return
+    check_mix(mix_lib().msgl_mix_postnorm(x.data_ptr(), _p(x_out), _p(h_out), _p(y), parts, _p(gate), weight.data_ptr(),
+                                          float(alpha), float(eps), rows, W, _code(weight), _stream()), "postnorm")
+
+
+def latent_prep(proj: torch.Tensor, q_abs: torch.Tensor, cache: Optional[torch.Tensor], out_loc: Optional[torch.Tensor],
+                positions: torch.Tensor, cos_sin: torch.Tensor, c_norm_w: Optional[torch.Tensor], eps: float, H: int, d: int,
+                r: int, R: int) -> None:
+    """Rotates the query parts into q_abs[:, :, R:]; with `cache`, norms + rotates + stores this layer's own latent rows."""
+    _dev(proj, q_abs, cache, out_loc, positions, cos_sin, c_norm_w)
+    T = proj.shape[0]
+    has_kv = cache is not None
+    assert proj.dim() == 2 and proj.stride(1) == 1
+    assert q_abs.dtype == torch.float32 and q_abs.is_contiguous() and q_abs.shape == (T, H, R + r)
+    assert cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.dim() == 2
+    if has_kv:
+        assert cache.is_contiguous() and cache.shape[1] == R + r and cache.dtype == proj.dtype
+        assert c_norm_w.dtype == proj.dtype and c_norm_w.shape == (R,) and out_loc.shape[0] == T
+    check_mix(mix_lib().msgl_mix_latent_prep(
+        proj.data_ptr(), proj.stride(0), q_abs.data_ptr(), _p(cache), _p(None if out_loc is None else _i32(out_loc)),
+        _i32(positions).data_ptr(), cos_sin.data_ptr(), _p(c_norm_w), float(eps), T, H, d, r, cos_sin.shape[1], R, int(has_kv),
+        _code(proj), _stream()), "latent_prep")
+
+
+def latent_attn(out: torch.Tensor, q_abs: torch.Tensor, cache: torch.Tensor, table: torch.Tensor, req_rows: torch.Tensor,
+                seq_lens: torch.Tensor, cu_q: torch.Tensor, batch: int, dv: int, scale: float) -> None:
+    _dev(out, q_abs, cache, table, req_rows, seq_lens, cu_q)
+    T, H, dk = q_abs.shape
+    assert q_abs.dtype == torch.float32 and q_abs.is_contiguous() and out.dtype == torch.float32 and out.is_contiguous()
+    assert out.shape == (T, H, dv) and cache.is_contiguous() and cache.shape[1] == dk
+    assert table.dtype == torch.int32 and table.stride(1) == 1
+    assert req_rows.numel() >= batch and seq_lens.numel() >= batch and cu_q.numel() >= batch + 1
+    check_mix(mix_lib().msgl_mix_latent_attn(
+        out.data_ptr(), q_abs.data_ptr(), cache.data_ptr(), table.data_ptr(), table.stride(0), _i32(req_rows).data_ptr(),
+        _i32(seq_lens).data_ptr(), _i32(cu_q).data_ptr(), batch, T, H, dk, dv, float(scale), _code(cache), _stream()), "latent_attn")
+
+
+def lightning(out: torch.Tensor, qkv: torch.Tensor, state: torch.Tensor, decay: torch.Tensor, cu_q: torch.Tensor,
+              seq_lens: torch.Tensor, slots: torch.Tensor, batch: int) -> None:
+    """state: fp32 [slots, H, d, dv]; qkv rows = [q H*d | k H*d | v H*dv | anything]."""
+    _dev(out, qkv, state, decay, cu_q, seq_lens, slots)
+    _, H, d, dv = state.shape
+    assert state.dtype == torch.float32 and state.is_contiguous() and decay.dtype == torch.float32 and decay.shape == (H,)
+    assert out.dtype == torch.float32 and out.is_contiguous() and out.shape == (qkv.shape[0], H * dv) and qkv.stride(1) == 1
+    check_mix(mix_lib().msgl_mix_lightning(
+        out.data_ptr(), qkv.data_ptr(), qkv.stride(0), state.data_ptr(), decay.data_ptr(), _i32(cu_q).data_ptr(),
+        _i32(seq_lens).data_ptr(), _i32(slots).data_ptr(), batch, H, d, dv, _code(qkv), _stream()), "lightning")
+
+
+def gated_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    _dev(o, gate, weight)
+    rows, N = o.shape
+    assert o.dtype == torch.float32 and o.is_contiguous() and gate.shape == (rows, N) and gate.stride(1) == 1
+    assert weight.dtype == gate.dtype and weight.shape == (N,) and weight.is_contiguous()
+    out = torch.empty((rows, N), dtype=gate.dtype, device=o.device)
+    check_mix(mix_lib().msgl_mix_gated_norm(out.data_ptr(), o.data_ptr(), gate.data_ptr(), gate.stride(0), weight.data_ptr(),
+                                            float(eps), rows, N, _code(gate), _stream()), "gated_norm")
+    return out
+
+
+def route(h: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int, groups: int, keep: int):
+    """-> (expert ids int32 [T, top], weights fp32 [T, top])."""
+    _dev(h, router, bias)
+    T, W = h.shape
+    E = router.shape[0]
+    assert h.is_contiguous() and router.is_contiguous() and router.shape == (E, W) and router.dtype == h.dtype
+    assert bias is None or (bias.dtype == h.dtype and bias.shape == (E,) and bias.is_contiguous())
+    ids = torch.empty((T, top), dtype=torch.int32, device=h.device)
+    wts = torch.empty((T, top), dtype=torch.float32, device=h.device)
+    check_mix(mix_lib().msgl_mix_route(ids.data_ptr(), wts.data_ptr(), h.data_ptr(), router.data_ptr(), _p(bias), T, W, E, top,
+                                       groups, keep, _code(h), _stream()), "route")
+    return ids, wts
+
+
+def moe_sort(ids: torch.Tensor, experts: int):
+    """-> (segment offsets int32 [E + 1], permutation int32 [T * top])."""
+    _dev(ids)
+    n = ids.numel()
+    seg = torch.empty(experts + 1, dtype=torch.int32, device=ids.device)
+    perm = torch.empty(max(n, 1), dtype=torch.int32, device=ids.device)
+    check_mix(mix_lib().msgl_mix_moe_sort(seg.data_ptr(), perm.data_ptr(), _i32(ids).data_ptr(), n, experts, _stream()), "moe_sort")
+    return seg, perm
+
+
+def gemm_nt(C: torch.Tensor, A: torch.Tensor, B: torch.Tensor, M: int, N: int, K: int, *, lda: int, ldb: int, ldc: int,
+            groups: int = 1, a_gs: int = 0, b_gs: int = 0, c_gs: int = 0, seg: Optional[torch.Tensor] = None,
+            a_rows: Optional[torch.Tensor] = None, a_div: int = 1, c_rows: Optional[torch.Tensor] = None,
+            act: int = ACT_NONE) -> None:
+    """The grouped / segmented / gathered product of csrc/seqmix.hip; the caller states every stride (elements)."""
+    _dev(C, A, B, seg, a_rows, c_rows)
+    check_mix(mix_lib().msgl_mix_gemm_nt(
+        C.data_ptr(), A.data_ptr(), B.data_ptr(), M, N, K, lda, ldb, ldc, groups, a_gs, b_gs, c_gs, _p(seg), _p(a_rows), a_div,
+        _p(c_rows), act, _code(A), _code(B), _code(C), _stream()), "gemm_nt")
+
+
+_NO_LIBRARY_SOLUTION: set = set()
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[M, N] = x[M, K] w[N, K]^T, fp32 accumulation, output in x's dtype."""
+    _dev(x, w)
+    assert x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1] and x.dtype == w.dtype
+    assert x.stride(1) == 1 and w.stride(1) == 1
+    M, K = x.shape
+    N = w.shape[0]
+    if out is None:
+        out = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    if M == 0:
+        return out
+    key = (M, N, K, x.stride(0), w.stride(0), out.stride(0), x.dtype)
+    if key not in _NO_LIBRARY_SOLUTION:
+        try:
+            if x.dtype == torch.float32:
+                ws = ops.gemm_workspace(x.device)
+                _lib.check_gemm(_lib.gemm_lib().msgl_gemm_nt(
+                    out.data_ptr(), x.data_ptr(), w.data_ptr(), M, N, K, x.stride(0), w.stride(0), out.stride(0), _lib.F32,
+                    ws.data_ptr(), ws.numel(), _stream()), "gemm_nt (fp32)")
+                return out
+            return ops.linear(x, w, out=out)
+        except _lib.MsglError:
+            _NO_LIBRARY_SOLUTION.add(key)
+    gemm_nt(out, x, w, M, N, K, lda=x.stride(0), ldb=w.stride(0), ldc=out.stride(0))
+    return out

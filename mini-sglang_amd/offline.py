@@ -261,3 +261,54 @@ class OfflineRunner:
         """Generated token ids of a (finished or running) request, read back from the token pool."""
         n_out = st.req.device_len - st.prompt_len
         return self.token_pool[st.req.table_idx, st.prompt_len: st.prompt_len + n_out].cpu().tolist()
+
+
+class StepReplayer:
+    """Feeds GIVEN tokens through the engine step by step and hands back logits instead of drawing tokens: the driver behind
+    trace replay and scoring.  A step is one batch of the engine's own forward: every entry brings a request's next tokens
+    (a portion of a prompt or a single token), requests are admitted at their first entry (page-table row = state slot from
+    the runner's free list, pages from its allocator), may sit out steps, and give row and pages back when they end."""
+
+    def __init__(self, engine: Engine, seed: Optional[int] = None) -> None:
+        self.engine = engine
+        self.runner = OfflineRunner(engine, seed=seed)
+        self.live: Dict[str, Req] = {}
+
+    def step(self, entries: Sequence[dict], end: Sequence[str] = ()) -> Optional[torch.Tensor]:
+        """entries: [{"id", "tokens", "want"}] -> logits [sum of wants, vocab] (device, model dtype) in entry order, or None
+        when nothing was asked for (the forward still runs: cache and state advance)."""
+        eng, run = self.engine, self.runner
+        reqs: List[Req] = []
+        rows: List[int] = []
+        off = 0
+        for e in entries:
+            toks = list(e["tokens"])
+            if not toks:
+                continue
+            ids = torch.tensor(toks, dtype=torch.int32)
+            req = self.live.get(e["id"])
+            if req is None:
+                if not run.free_rows:
+                    raise RuntimeError("no free request row: more live requests than max_running_req")
+                row = run.free_rows.pop()
+                req = Req(input_ids=ids, table_idx=row, cached_len=0, output_len=0, uid=row, sampling_params=SamplingParams())
+                req.max_device_len = eng.max_seq_len
+                self.live[e["id"]] = req
+            else:
+                req.device_len = req.cached_len + len(toks)
+            if req.device_len > eng.max_seq_len:
+                raise RuntimeError(f"request {e['id']!r} grows to {req.device_len} tokens, above the engine's {eng.max_seq_len}")
+            run.token_pool[req.table_idx, req.cached_len: req.device_len] = ids.pin_memory().to(run.device, non_blocking=True)
+            reqs.append(req)
+            rows += [off + int(w) for w in e.get("want", ())]
+            off += len(toks)
+        logits = None
+        if reqs:
+            batch, _ = run._make_batch(reqs, "prefill")
+            batch.logit_rows = torch.tensor(rows, dtype=torch.int32).pin_memory().to(run.device, non_blocking=True)
+            logits = eng.forward_logits(batch)
+        for rid in end:
+            req = self.live.pop(rid, None)
+            if req is not None:
+                run._free(req)
+        return logits if rows else None
