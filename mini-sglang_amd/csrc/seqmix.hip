@@ -284,12 +284,15 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(float* __restrict__ ou
 }
 
 // ------------------------------------------------------------------------------------------------ lightning recurrence
-// Workgroup = one (head, request).  Thread (column v, slice s) keeps rows s, s + NS, ... of column v of the d x dv state in
-// registers.  Tokens go through in batches of kLtTok: q, k, v rows staged in LDS (SiLU applied in fp32), every thread walks
-// the batch sequentially (S <- decay S + k v^T, partial o = sum over its rows of S q), the NS partials of a column are
-// added in slice order.  A request that starts at position 0 starts from a zero state; the state row is the request's slot.
+// Workgroup = one (head, request, block of CB state columns): columns of the d x dv state never mix (o[v] = sum_r S[r][v] q[r]),
+// so they spread over workgroups freely.  Thread (column v, slice s) keeps rows s, s + NS, ... of column v in registers.
+// Tokens go through in batches of kLtTok: q, k, v rows staged in LDS (SiLU applied in fp32), every thread walks the batch
+// sequentially (S <- decay S + k v^T, partial o = sum over its rows of S q), the NS partials of a column are added in slice
+// order.  A request that starts at position 0 starts from a zero state; the state row is the request's slot.  The arithmetic
+// of a token does not depend on where a portion starts or ends: cutting a prompt anywhere gives the same bits.
 constexpr int kLtTok = 16;
 constexpr int kLtMaxRows = 64;
+constexpr int kLtMaxCols = 64;
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
@@ -297,18 +300,20 @@ template <typename T>
 __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out, const T* __restrict__ qkv, int64_t ld_qkv,
                                                         float* __restrict__ state, const float* __restrict__ decay,
                                                         const int* __restrict__ cu_q, const int* __restrict__ seq_lens,
-                                                        const int* __restrict__ slots, int H, int d, int dv, int NS) {
+                                                        const int* __restrict__ slots, int H, int d, int dv, int CB, int NS) {
   extern __shared__ float lds[];
   float* sq = lds;                    // [kLtTok][d]
   float* skk = sq + kLtTok * d;       // [kLtTok][d]
-  float* sv = skk + kLtTok * d;       // [kLtTok][dv]
-  float* part = sv + kLtTok * dv;     // [kLtTok][NS][dv]
-  const int hh = blockIdx.x, b = blockIdx.y;
+  float* sv = skk + kLtTok * d;       // [kLtTok][CB]
+  float* part = sv + kLtTok * CB;     // [kLtTok][NS][CB]
+  const int hh = blockIdx.x, b = blockIdx.y, v0 = blockIdx.z * CB;
   const int t0 = cu_q[b], n = cu_q[b + 1] - t0;
   if (n <= 0) return;
   const bool fresh = seq_lens[b] - n == 0;
-  const int v = threadIdx.x % dv, s = threadIdx.x / dv;
-  const bool active = s < NS;
+  const int vl = threadIdx.x % CB, s = threadIdx.x / CB;
+  const int v = v0 + vl;
+  const int nc = min(CB, dv - v0);  // columns of this block
+  const bool active = s < NS && v < dv;
   float* S = state + ((size_t)slots[b] * H + hh) * d * dv;
   const float dec = decay[hh];
   float reg[kLtMaxRows];
@@ -317,7 +322,7 @@ __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out,
     const int row = s + i * NS;
     reg[i] = (active && row < d && !fresh) ? S[(size_t)row * dv + v] : 0.f;
   }
-  const int64_t qo = (int64_t)hh * d, ko = (int64_t)H * d + (int64_t)hh * d, vo = 2 * (int64_t)H * d + (int64_t)hh * dv;
+  const int64_t qo = (int64_t)hh * d, ko = (int64_t)H * d + (int64_t)hh * d, vo = 2 * (int64_t)H * d + (int64_t)hh * dv + v0;
   for (int c0 = 0; c0 < n; c0 += kLtTok) {
     const int nt = min(kLtTok, n - c0);
     __syncthreads();
@@ -327,14 +332,14 @@ __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out,
       sq[tt * d + i] = silu_f(ld(row + qo + i));
       skk[tt * d + i] = silu_f(ld(row + ko + i));
     }
-    for (int e = threadIdx.x; e < nt * dv; e += 256) {
-      const int tt = e / dv, i = e - tt * dv;
-      sv[tt * dv + i] = silu_f(ld(qkv + (size_t)(t0 + c0 + tt) * ld_qkv + vo + i));
+    for (int e = threadIdx.x; e < nt * nc; e += 256) {
+      const int tt = e / nc, i = e - tt * nc;
+      sv[tt * CB + i] = silu_f(ld(qkv + (size_t)(t0 + c0 + tt) * ld_qkv + vo + i));
     }
     __syncthreads();
     if (active) {
       for (int tt = 0; tt < nt; ++tt) {
-        const float vv = sv[tt * dv + v];
+        const float vv = sv[tt * CB + vl];
         float acc = 0.f;
 #pragma unroll
         for (int i = 0; i < kLtMaxRows; ++i) {
@@ -344,15 +349,15 @@ __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out,
             acc = fmaf(reg[i], sq[tt * d + row], acc);
           }
         }
-        part[(tt * NS + s) * dv + v] = acc;
+        part[(tt * NS + s) * CB + vl] = acc;
       }
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < nt * dv; e += 256) {
-      const int tt = e / dv, i = e - tt * dv;
+    for (int e = threadIdx.x; e < nt * nc; e += 256) {
+      const int tt = e / nc, i = e - tt * nc;
       float acc = 0.f;
-      for (int k = 0; k < NS; ++k) acc += part[(tt * NS + k) * dv + i];
-      out[(size_t)(t0 + c0 + tt) * ((size_t)H * dv) + (size_t)hh * dv + i] = acc;
+      for (int k = 0; k < NS; ++k) acc += part[(tt * NS + k) * CB + i];
+      out[(size_t)(t0 + c0 + tt) * ((size_t)H * dv) + (size_t)hh * dv + v0 + i] = acc;
     }
   }
   if (active) {
@@ -651,15 +656,18 @@ int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, cons
 int msgl_mix_lightning(float* out, const void* qkv, int64_t ld_qkv, float* state, const float* decay, const int* cu_q, const int* seq_lens,
                        const int* slots, int batch, int H, int d, int dv, int dtype, void* stream) {
   MIX_REQUIRE(out && qkv && state && decay && cu_q && seq_lens && slots && dtype_ok(dtype), "lightning: null pointer / dtype");
-  MIX_REQUIRE(batch >= 1 && H >= 1 && d >= 1 && dv >= 1 && dv <= 256, "lightning: bad sizes (value width %d, at most 256)", dv);
+  MIX_REQUIRE(batch >= 1 && batch <= 65535 && H >= 1 && d >= 1 && dv >= 1, "lightning: bad sizes");
   MIX_REQUIRE(ld_qkv >= (int64_t)H * (2 * d + dv), "lightning: projection row too short");
-  const int NS = 256 / dv;
-  MIX_REQUIRE((d + NS - 1) / NS <= kLtMaxRows, "lightning: state %d x %d needs more than %d rows per thread", d, dv, kLtMaxRows);
-  const size_t lds = (size_t)(kLtTok * (2 * d + dv) + kLtTok * NS * dv) * sizeof(float);
+  const int CB = dv < kLtMaxCols ? dv : kLtMaxCols;
+  const int NS = 256 / CB;
+  MIX_REQUIRE((d + NS - 1) / NS <= kLtMaxRows, "lightning: key size %d needs more than %d state rows per thread", d, kLtMaxRows);
+  const int col_blocks = (dv + CB - 1) / CB;
+  MIX_REQUIRE(col_blocks <= 65535, "lightning: value width %d", dv);
+  const size_t lds = (size_t)(kLtTok * (2 * d + CB) + kLtTok * NS * CB) * sizeof(float);
   hipStream_t s = static_cast<hipStream_t>(stream);
   DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)lightning_kernel<T>, lds) == 0, "lightning: LDS request refused");
-             hipLaunchKernelGGL(lightning_kernel<T>, dim3(H, batch), dim3(256), lds, s, out, cp<T>(qkv), ld_qkv, state, decay, cu_q,
-                                seq_lens, slots, H, d, dv, NS);)
+             hipLaunchKernelGGL(lightning_kernel<T>, dim3(H, batch, col_blocks), dim3(256), lds, s, out, cp<T>(qkv), ld_qkv, state, decay,
+                                cu_q, seq_lens, slots, H, d, dv, CB, NS);)
   MIX_LAUNCHED("lightning");
   return MSGL_MIX_OK;
 }

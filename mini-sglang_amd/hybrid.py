@@ -224,6 +224,9 @@ class HybridDecoder:
                 put(L.w_in, torch.cat([state[p + "q"], state[p + "k"], state[p + "v"], state[p + "g"]], dim=0))
                 put(L.out_norm, state[p + "norm"])
             put(L.o, state[p + "o"])
+            if s.mlp is None and f"l{i}.norm2" in state:  # a layer without feed-forward that still norms a second time
+                L.norm2 = torch.empty_like(L.norm1)
+                put(L.norm2, state[f"l{i}.norm2"])
             if s.mlp is not None:
                 q = f"l{i}.mlp."
                 put(L.norm2, state[f"l{i}.norm2"])
@@ -254,6 +257,8 @@ class HybridDecoder:
                 out[p + "q"], out[p + "k"], out[p + "v"], out[p + "g"] = L.w_in[:a], L.w_in[a:2 * a], L.w_in[2 * a:2 * a + b], L.w_in[2 * a + b:]
                 out[p + "norm"] = L.out_norm
             out[p + "o"] = L.o
+            if s.mlp is None and L.norm2 is not None:
+                out[f"l{i}.norm2"] = L.norm2
             if s.mlp is not None:
                 q = f"l{i}.mlp."
                 out[f"l{i}.norm2"], out[q + "router"] = L.norm2, L.router
@@ -318,6 +323,8 @@ class HybridDecoder:
             if L.spec.mlp is not None:
                 y, wts = self._experts(L, h)
                 mixops.postnorm(x, L.norm2, eps, y=y, gate=wts, alpha=alpha, x_out=x, h_out=h)
+            elif L.norm2 is not None:
+                mixops.postnorm(x, L.norm2, eps, alpha=alpha, x_out=x, h_out=h)
             if layer_outputs is not None:
                 layer_outputs.append(x.clone())
         rows = getattr(batch, "logit_rows", None)
