@@ -661,7 +661,17 @@ def main() -> None:
                     help="N > 1: time ONE rank's shard of a TP = N decode step on this GPU with the collectives looped back "
                          "(tools/rank_shard_bench.py): an upper bound on the TP = N speed-up before any link is paid")
     ap.add_argument("--tp1-ms", type=float, default=None, help="with --rank-shard: the TP1 ms/step to compare against")
+    ap.add_argument("--hybrid", action="store_true",
+                    help="instead of the default workload: prefill / decode throughput of the hybrid decoder (latent attention + "
+                         "lightning recurrence + routed experts) beside a dense decoder of equal size, and its kernels against "
+                         "their rooflines (tools/hybrid_bench.py; further flags after --hybrid-args)")
+    ap.add_argument("--hybrid-args", nargs=argparse.REMAINDER, default=[], help="flags handed to tools/hybrid_bench.py")
     args = ap.parse_args()
+    if args.hybrid:
+        from tools.hybrid_bench import main as hybrid_main
+
+        hybrid_main(list(args.hybrid_args))
+        return
     if args.rank_shard > 1:
         from tools.rank_shard_bench import main as rank_shard_main
 

@@ -558,6 +558,143 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(TC* __restrict__ C, const 
   }
 }
 
+// ------------------------------------------------------------------------------------------------ grouped GEMM on the matrix cores
+// The same contract as gemm_nt_kernel for 16-bit B (weights): A is rounded to bf16 on its way into LDS (it IS bf16 except for
+// the fp32 latent that meets W_uv), products on v_mfma_f32_16x16x32_bf16 with fp32 accumulation.  128 x 128 tile, 4 waves of
+// 64 x 64 (4 x 4 MFMA tiles each), k in steps of 32; the next step's global loads are issued before the current step's
+// MFMAs.  LDS rows are 40 elements apart (80 B): the 16 lanes of a fragment read land on 16 different bank quads.  A wave
+// whose rows lie past the end of a (short) expert segment skips its MFMAs, so a decode step pays for the weight stream only.
+// An output element's k order is fixed, wherever its row sits in a segment: results do not depend on the batch around it.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+struct __attribute__((aligned(16))) Q4 {
+  uint32_t x, y, z, w;
+};
+constexpr int kMT = 128, kMK = 32, kMLd = 40;
+
+__device__ __forceinline__ uint32_t bf16_bits(float v) {
+  bf16_t t;
+  st(&t, v);
+  return t.bits;
+}
+
+// eight consecutive k of one row as packed bf16; `n` of them exist (the rest read as zero); vec: 16-byte loads are legal
+__device__ __forceinline__ Q4 load8(const bf16_t* p, int n, bool vec) {
+  if (vec && n >= 8) return *reinterpret_cast<const Q4*>(p);
+  uint32_t e[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) e[i] = i < n ? p[i].bits : 0u;
+  return Q4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+}
+__device__ __forceinline__ Q4 load8(const float* p, int n, bool vec) {
+  float f[8];
+  if (vec && n >= 8) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = i < n ? p[i] : 0.f;
+  }
+  return Q4{bf16_bits(f[0]) | (bf16_bits(f[1]) << 16), bf16_bits(f[2]) | (bf16_bits(f[3]) << 16),
+            bf16_bits(f[4]) | (bf16_bits(f[5]) << 16), bf16_bits(f[6]) | (bf16_bits(f[7]) << 16)};
+}
+
+template <typename TA, typename TC>
+__global__ __launch_bounds__(256) void gemm_nt_mfma_kernel(TC* __restrict__ C, const TA* __restrict__ A, const bf16_t* __restrict__ Bm, int M,
+                                                           int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int64_t a_gs, int64_t b_gs,
+                                                           int64_t c_gs, const int* __restrict__ seg, const int* __restrict__ a_rows,
+                                                           int a_div, const int* __restrict__ c_rows, int act, int a_vec, int b_vec) {
+  __shared__ __attribute__((aligned(16))) uint16_t sa[kMT * kMLd];
+  __shared__ __attribute__((aligned(16))) uint16_t sb[kMT * kMLd];
+  const int g = blockIdx.z;
+  int row0 = 0, rows = M;
+  if (seg) {
+    row0 = seg[g];
+    rows = seg[g + 1] - row0;
+  }
+  const int m0 = blockIdx.y * kMT, n0 = blockIdx.x * kMT;
+  if (m0 >= rows) return;
+  const TA* Ag = A + (seg ? 0 : g * a_gs);
+  const bf16_t* Bg = Bm + g * b_gs;
+  TC* Cg = C + (seg ? 0 : g * c_gs);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int lr = threadIdx.x >> 2, ks = (threadIdx.x & 3) * 8;
+  int64_t a_off[2], b_off[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int ml = m0 + lr + 64 * u, n = n0 + lr + 64 * u;
+    a_off[u] = -1;
+    if (ml < rows) {
+      const int m = row0 + ml;
+      a_off[u] = (int64_t)(a_rows ? a_rows[m] / a_div : m) * lda;
+    }
+    b_off[u] = n < N ? (int64_t)n * ldb : -1;
+  }
+  Q4 ra[2], rb[2];
+  auto gload = [&](int k0) {
+    const int k = k0 + ks, n = K - k;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      ra[u] = (a_off[u] >= 0 && n > 0) ? load8(Ag + a_off[u] + k, n, a_vec != 0) : Q4{0u, 0u, 0u, 0u};
+      rb[u] = (b_off[u] >= 0 && n > 0) ? load8(Bg + b_off[u] + k, n, b_vec != 0) : Q4{0u, 0u, 0u, 0u};
+    }
+  };
+  f32x4_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int live_i = min(4, (rows - m0 - wm + 15) / 16);  // 16-row tiles of this wave that hold rows (<= 0: none)
+  gload(0);
+  for (int k0 = 0; k0 < K; k0 += kMK) {
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      *reinterpret_cast<Q4*>(&sa[(lr + 64 * u) * kMLd + ks]) = ra[u];
+      *reinterpret_cast<Q4*>(&sb[(lr + 64 * u) * kMLd + ks]) = rb[u];
+    }
+    __syncthreads();
+    if (k0 + kMK < K) gload(k0 + kMK);
+    if (live_i > 0) {
+      bf16x8_t fb[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        fb[j] = *reinterpret_cast<const bf16x8_t*>(&sb[(wn + j * 16 + (lane & 15)) * kMLd + (lane >> 4) * 8]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (i < live_i) {
+          const bf16x8_t fa = *reinterpret_cast<const bf16x8_t*>(&sa[(wm + i * 16 + (lane & 15)) * kMLd + (lane >> 4) * 8]);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j], fa, acc[i][j], 0, 0, 0);
+        }
+      }
+    }
+  }
+  // lane holds C[m = tile row (lane & 15)][n = 4 (lane >> 4) .. + 3] of every 16 x 16 tile
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int ml = m0 + wm + i * 16 + (lane & 15);
+    if (ml >= rows) continue;
+    const int m = row0 + ml;
+    const int64_t c_off = (int64_t)(c_rows ? c_rows[m] : m) * ldc;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int n = n0 + wn + j * 16 + 4 * (lane >> 4) + c;
+        if (n >= N) continue;
+        float v = acc[i][j][c];
+        if (act == MSGL_MIX_ACT_RELU2) {
+          v = fmaxf(v, 0.f);
+          v = v * v;
+        }
+        st(Cg + c_off + n, v);
+      }
+    }
+  }
+}
+
 template <typename T>
 const T* cp(const void* p) {
   return static_cast<const T*>(p);
@@ -713,9 +850,31 @@ int msgl_mix_gemm_nt(void* C, const void* A, const void* B, int M, int N, int K,
   MIX_REQUIRE(lda >= K && ldb >= K && a_div >= 1, "gemm_nt: leading dimensions");
   MIX_REQUIRE(act == MSGL_MIX_ACT_NONE || act == MSGL_MIX_ACT_RELU2, "gemm_nt: activation code %d", act);
   if (M == 0) return MSGL_MIX_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (tb == MSGL_MIX_BF16) {  // 16-bit weights: the matrix-core kernel
+    const int row_tiles = (M + kMT - 1) / kMT;
+    MIX_REQUIRE(row_tiles <= 65535, "gemm_nt: too many rows");
+    const dim3 grid((N + kMT - 1) / kMT, row_tiles, groups);
+    auto al = [](const void* p, int64_t ld, int64_t gs, int elems) {
+      return ((uintptr_t)p & 15u) == 0 && ld % elems == 0 && gs % elems == 0;
+    };
+    const int b_vec = al(B, ldb, b_gs, 8);
+    const int a_vec = ta == MSGL_MIX_BF16 ? al(A, lda, a_gs, 8) : al(A, lda, a_gs, 4);
+#define MFMA_CASE(CA, CC, TA, TC)                                                                                                   \
+  if (ta == CA && tc == CC) {                                                                                                       \
+    hipLaunchKernelGGL((gemm_nt_mfma_kernel<TA, TC>), grid, dim3(256), 0, s, mp<TC>(C), cp<TA>(A), cp<bf16_t>(B), M, N, K, lda, ldb, \
+                       ldc, a_gs, b_gs, c_gs, seg, a_rows, a_div, c_rows, act, a_vec, b_vec);                                       \
+    MIX_LAUNCHED("gemm_nt (matrix cores)");                                                                                         \
+    return MSGL_MIX_OK;                                                                                                             \
+  }
+    MFMA_CASE(MSGL_MIX_BF16, MSGL_MIX_BF16, bf16_t, bf16_t)
+    MFMA_CASE(MSGL_MIX_BF16, MSGL_MIX_F32, bf16_t, float)
+    MFMA_CASE(MSGL_MIX_F32, MSGL_MIX_BF16, float, bf16_t)
+    MFMA_CASE(MSGL_MIX_F32, MSGL_MIX_F32, float, float)
+#undef MFMA_CASE
+  }
   const int row_tiles = (M + kTile - 1) / kTile;
   MIX_REQUIRE(row_tiles <= 65535, "gemm_nt: too many rows");
-  hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((N + kTile - 1) / kTile, row_tiles, groups);
 #define GEMM_CASE(CA, CB, CC, TA, TB, TC)                                                                                            \
   if (ta == CA && tb == CB && tc == CC) {                                                                                            \
@@ -724,9 +883,6 @@ int msgl_mix_gemm_nt(void* C, const void* A, const void* B, int M, int N, int K,
     MIX_LAUNCHED("gemm_nt");                                                                                                         \
     return MSGL_MIX_OK;                                                                                                              \
   }
-  GEMM_CASE(MSGL_MIX_BF16, MSGL_MIX_BF16, MSGL_MIX_BF16, bf16_t, bf16_t, bf16_t)
-  GEMM_CASE(MSGL_MIX_BF16, MSGL_MIX_BF16, MSGL_MIX_F32, bf16_t, bf16_t, float)
-  GEMM_CASE(MSGL_MIX_F32, MSGL_MIX_BF16, MSGL_MIX_BF16, float, bf16_t, bf16_t)
   GEMM_CASE(MSGL_MIX_F32, MSGL_MIX_F32, MSGL_MIX_F32, float, float, float)
 #undef GEMM_CASE
   set_err("gemm_nt: no kernel for dtype codes (%d, %d, %d)", ta, tb, tc);

@@ -217,6 +217,55 @@ def test_grouped_product_and_bucketing(dev):
             assert torch.allclose(y[t, k].cpu().double(), down[e].double() @ a, rtol=1e-4, atol=1e-3)
 
 
+@pytest.mark.parametrize("M,N,K", [(70, 50, 37), (200, 256, 64), (1, 130, 96), (129, 127, 264)])
+@pytest.mark.parametrize("a_dtype,c_dtype", [(torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                             (torch.float32, torch.bfloat16)], ids=["bf16", "bf16-to-fp32", "fp32-a"])
+def test_matrix_core_product(dev, M, N, K, a_dtype, c_dtype):
+    """16-bit weights take the matrix-core kernel: sizes off every tile and vector boundary, per-head groups laid out side by
+    side in one row (the latent-attention products), fp32 left operand rounded on the way in."""
+    from mini_sglang_amd import mixops
+
+    torch.manual_seed(M + N + K)
+    G = 3
+    a = torch.randn(M, G * K + 5).to(a_dtype)
+    b = torch.randn(G, N, K).to(torch.bfloat16)
+    c = torch.zeros(M, G * N + 3, dtype=c_dtype, device=dev)
+    mixops.gemm_nt(c, a.to(dev), b.to(dev), M, N, K, lda=a.stride(0), ldb=K, ldc=c.stride(0), groups=G, a_gs=K, b_gs=N * K, c_gs=N)
+    for g in range(G):
+        ag = a[:, g * K: (g + 1) * K].to(torch.bfloat16).double()
+        ref = ag @ b[g].double().T
+        got = c[:, g * N: (g + 1) * N].cpu().double()
+        tol = 2e-2 if c_dtype == torch.bfloat16 else 1e-4
+        assert float((got - ref).abs().max() / ref.abs().max()) < tol, g
+    assert float(c[:, G * N:].abs().max()) == 0.0
+
+
+def test_expert_products_bf16(dev):
+    """The expert path in 16 bits (matrix cores, gathered rows in, scattered rows out, ReLU^2 between), segments of very
+    unequal length including empty ones."""
+    from mini_sglang_amd import mixops
+
+    torch.manual_seed(3)
+    T, top, E, W, F = 300, 2, 7, 72, 136
+    ids = torch.randint(0, 3, (T, top), dtype=torch.int32)
+    ids[:5, 0] = 6  # expert 6: five rows; experts 3..5: none
+    seg, perm = mixops.moe_sort(ids.to(dev), E)
+    h = torch.randn(T, W).to(torch.bfloat16)
+    up, down = (torch.randn(E, F, W) * W ** -0.5).to(torch.bfloat16), (torch.randn(E, W, F) * F ** -0.5).to(torch.bfloat16)
+    act = torch.zeros(T * top, F, dtype=torch.bfloat16, device=dev)
+    mixops.gemm_nt(act, h.to(dev), up.to(dev), T * top, F, W, lda=W, ldb=W, ldc=F, groups=E, b_gs=F * W, seg=seg, a_rows=perm,
+                   a_div=top, act=mixops.ACT_RELU2)
+    y = torch.zeros(T, top, W, dtype=torch.bfloat16, device=dev)
+    mixops.gemm_nt(y, act, down.to(dev), T * top, W, F, lda=F, ldb=F, ldc=W, groups=E, b_gs=W * F, seg=seg, c_rows=perm)
+    yh = y.cpu().double()
+    for t in range(0, T, 7):
+        for k in range(top):
+            e = int(ids[t, k])
+            a = (torch.relu(up[e].double() @ h[t].double()) ** 2).to(torch.bfloat16).double()
+            ref = down[e].double() @ a
+            assert float((yh[t, k] - ref).abs().max()) < 2e-2 * float(ref.abs().max()) + 1e-3, (t, k)
+
+
 @pytest.mark.parametrize("n_keys", [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 300])
 def test_latent_attention_far_key_takes_all(dev, n_keys):
     """One key far back (the first, or one on a page border) is made to win the softmax for one head while another head
