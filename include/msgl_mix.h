@@ -51,10 +51,15 @@ int msgl_mix_latent_prep(const void* proj, int64_t ld_proj, float* q_abs, void* 
 /* Causal attention of H heads over ONE shared key row per token: score = q_abs[t, h] . cache[slot] * scale over dk entries,
  * softmax in fp32, out[t, h] = sum_j p_j cache[slot_j][0 : dv] (fp32).  Requests as in the paged backend: table rows of token
  * slots, seq_lens = keys after this forward, cu_q = exclusive prefix of new tokens; prefill portions, single decoded tokens
- * and any mix of them in one launch. */
+ * and any mix of them in one launch.
+ * bf16 caches run on the matrix cores (Q and the softmax weights rounded to bf16 for the two products, fp32 accumulation and fp32
+ * softmax); `splits` > 1 cuts every request's keys into that many ranges whose partial results (workspace: fp32,
+ * msgl_mix_latent_attn_workspace_floats) a second launch merges -- for steps with few query rows and many keys.  fp32 caches
+ * take the plain fp32 kernel (splits is ignored). */
+int msgl_mix_latent_attn_workspace_floats(int total_q, int H, int dv, int splits);
 int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, const int* table, int64_t table_stride, const int* req_rows,
                          const int* seq_lens, const int* cu_q, int batch, int total_q, int H, int dk, int dv, float scale, int dtype,
-                         void* stream);
+                         int splits, float* workspace, void* stream);
 
 /* Linear recurrence per (request, head): S <- decay[h] S + k v^T, out = S^T q, with q, k, v = SiLU of the projection row
  * [q: H x d | k: H x d | v: H x dv | ...].  state: fp32 [slots, H, d, dv], row slots[b]; a request whose first new token is at

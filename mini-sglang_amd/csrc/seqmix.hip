@@ -695,6 +695,188 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma_kernel(TC* __restrict__ C, c
   }
 }
 
+// ------------------------------------------------------------------------------------------------ latent attention on the matrix cores
+// bf16 caches.  A workgroup = 64 query rows ((token, head) pairs of one request: QT tokens x HB heads) in 4 waves of 16 rows,
+// one key range (split z of the keys its last token sees).  Keys come through LDS in tiles of 32 rows, row-major, 16-byte
+// padded (fragment reads of 16 rows hit 16 different bank quads).  Per 16-key subtile and wave:
+//   S^T[16 keys x 16 rows] = K . Q^T     KC x v_mfma_f32_16x16x32_bf16   (Q fragments live in registers, rounded to bf16 once)
+//   a lane then holds ONE query row and FOUR keys: the B-operand layout of the second product, so P stays in its lane;
+//   O^T[16 v x 16 rows] += V^T . P^T     VC x v_mfma_f32_16x16x16_bf16, V^T fragments read TRANSPOSED out of the same row-major
+//   key tile (the latent is both key and value): in a 16-lane group, source lane s points at row 4 g + s / 4, columns
+//   4 (s % 4) .. + 3 and ds_read_b64_tr_b16 hands lane j the four keys of column j.
+// Softmax in fp32 per row: tile max across the four lane groups, running (m, l), O rescaled when a row's max moved.
+// splits > 1 (decode: few rows, many keys): (m, l, O) partials per split, merged by latent_attn_merge_kernel.
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((address_space(3))) s16x4_t lds_s16x4_t;
+constexpr int kAKT = 32;
+
+template <int KC, int VC>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+                                                               const float* __restrict__ q_abs, const bf16_t* __restrict__ cache,
+                                                               const int* __restrict__ table, int64_t table_stride,
+                                                               const int* __restrict__ req_rows, const int* __restrict__ seq_lens,
+                                                               const int* __restrict__ cu_q, int B, int H, int dk, int dv, float scale,
+                                                               int QT, int HB, int splits, int vec) {
+  constexpr int KS = KC * 32 + 8;
+  __shared__ __attribute__((aligned(16))) uint16_t sk[kAKT * KS];
+  __shared__ int s_req, s_tok0;
+  if (threadIdx.x == 0) {
+    int g = blockIdx.x, found = -1, tok0 = 0;
+    for (int b = 0; b < B; ++b) {
+      const int n = cu_q[b + 1] - cu_q[b];
+      const int groups = (n + QT - 1) / QT;
+      if (g < groups) {
+        found = b;
+        tok0 = g * QT;
+        break;
+      }
+      g -= groups;
+    }
+    s_req = found;
+    s_tok0 = tok0;
+  }
+  __syncthreads();
+  const int b = s_req;
+  if (b < 0) return;
+  const int q_len = cu_q[b + 1] - cu_q[b];
+  const int start = seq_lens[b] - q_len;
+  const int h0 = blockIdx.y * HB, z = blockIdx.z;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const int r = wave * 16 + lr;
+  const int tl = s_tok0 + r / HB, hh = h0 + r % HB;
+  const bool valid = r < QT * HB && tl < q_len && hh < H;
+  const int tok = cu_q[b] + (valid ? tl : s_tok0);
+  const int head = valid ? hh : h0;
+  const int limit = valid ? start + tl : -1;
+  const int last_tok = min(s_tok0 + QT, q_len) - 1;
+  const int n_keys = start + last_tok + 1;
+  const int per = ((n_keys + splits - 1) / splits + kAKT - 1) / kAKT * kAKT;
+  const int k_begin = z * per, k_end = min(n_keys, k_begin + per);
+  const bool wave_live = __builtin_amdgcn_ballot_w64(valid) != 0;
+  // query fragments: row lr of this wave, k = 32 kc + 8 lg .. + 7
+  bf16x8_t qf[KC];
+  {
+    const float* qrow = q_abs + ((size_t)tok * H + head) * dk;
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) {
+      const int k = kc * 32 + lg * 8;
+      Q4 v = (valid && k < dk) ? load8(qrow + k, dk - k, (dk & 3) == 0) : Q4{0u, 0u, 0u, 0u};
+      qf[kc] = __builtin_bit_cast(bf16x8_t, v);
+    }
+  }
+  f32x4_t o[VC];
+#pragma unroll
+  for (int vt = 0; vt < VC; ++vt) o[vt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, lsum = 0.f;
+  const int* trow = table + (size_t)req_rows[b] * table_stride;
+  for (int j0 = k_begin; j0 < k_end; j0 += kAKT) {
+    __syncthreads();
+    for (int e = threadIdx.x; e < kAKT * KC * 4; e += 256) {
+      const int key = e / (KC * 4), ch = e - key * (KC * 4);
+      const int j = j0 + key, k = ch * 8;
+      Q4 v{0u, 0u, 0u, 0u};
+      if (j < k_end && k < dk) v = load8(cache + (size_t)trow[j] * dk + k, dk - k, vec != 0);
+      *reinterpret_cast<Q4*>(&sk[key * KS + k]) = v;
+    }
+    __syncthreads();
+    if (!wave_live) continue;
+#pragma unroll
+    for (int ks = 0; ks < kAKT / 16; ++ks) {
+      if (j0 + ks * 16 >= k_end) break;
+      f32x4_t sacc{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kc = 0; kc < KC; ++kc) {
+        const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(&sk[(ks * 16 + lr) * KS + kc * 32 + lg * 8]);
+        sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kc], sacc, 0, 0, 0);
+      }
+      float sc[4], mx = -INFINITY;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int j = j0 + ks * 16 + 4 * lg + c;
+        sc[c] = (j <= limit && j < k_end) ? sacc[c] * scale : -INFINITY;
+        mx = fmaxf(mx, sc[c]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m, mx);
+      const bool none = m_new == -INFINITY;  // this row has seen no key yet
+      const float corr = none ? 1.f : __expf(m - m_new);
+      float pe[4], ps = 0.f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        pe[c] = none ? 0.f : __expf(sc[c] - m_new);
+        ps += pe[c];
+      }
+      lsum = lsum * corr + ps;
+      m = m_new;
+      if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {
+#pragma unroll
+        for (int vt = 0; vt < VC; ++vt) {
+          o[vt][0] *= corr; o[vt][1] *= corr; o[vt][2] *= corr; o[vt][3] *= corr;
+        }
+      }
+      const uint32_t p01 = bf16_bits(pe[0]) | (bf16_bits(pe[1]) << 16), p23 = bf16_bits(pe[2]) | (bf16_bits(pe[3]) << 16);
+      const s16x4_t pf = __builtin_bit_cast(s16x4_t, uint2{p01, p23});
+      const uint16_t* vbase = &sk[(ks * 16 + 4 * lg + (lr >> 2)) * KS + 4 * (lr & 3)];
+#pragma unroll
+      for (int vt = 0; vt < VC; ++vt) {
+        const s16x4_t vf = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(vbase + vt * 16));
+        o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pf, o[vt], 0, 0, 0);
+      }
+    }
+  }
+  lsum += __shfl_xor(lsum, 16, 64);
+  lsum += __shfl_xor(lsum, 32, 64);
+  if (!valid) return;
+  const size_t row = (size_t)tok * H + head;
+  if (splits == 1) {
+    const float inv = 1.0f / lsum;
+#pragma unroll
+    for (int vt = 0; vt < VC; ++vt)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int v = vt * 16 + 4 * lg + c;
+        if (v < dv) out[row * dv + v] = o[vt][c] * inv;
+      }
+  } else {
+    float* po = part_o + (row * splits + z) * dv;
+#pragma unroll
+    for (int vt = 0; vt < VC; ++vt)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int v = vt * 16 + 4 * lg + c;
+        if (v < dv) po[v] = o[vt][c];
+      }
+    if (lg == 0) {
+      part_ml[(row * splits + z) * 2] = m;
+      part_ml[(row * splits + z) * 2 + 1] = lsum;
+    }
+  }
+}
+
+// out[row] = sum_z e^(m_z - m*) o_z / sum_z e^(m_z - m*) l_z, splits in order; a split without keys has l = 0 and m = -inf
+__global__ __launch_bounds__(64) void latent_attn_merge_kernel(float* __restrict__ out, const float* __restrict__ part_o,
+                                                               const float* __restrict__ part_ml, int splits, int dv) {
+  const size_t row = blockIdx.x;
+  float ms = -INFINITY;
+  for (int z = 0; z < splits; ++z) ms = fmaxf(ms, part_ml[(row * splits + z) * 2]);
+  float l = 0.f;
+  for (int z = 0; z < splits; ++z) {
+    const float mz = part_ml[(row * splits + z) * 2];
+    if (mz > -INFINITY) l += part_ml[(row * splits + z) * 2 + 1] * __expf(mz - ms);
+  }
+  const float inv = 1.0f / l;
+  for (int v = threadIdx.x; v < dv; v += 64) {
+    float acc = 0.f;
+    for (int z = 0; z < splits; ++z) {
+      const float mz = part_ml[(row * splits + z) * 2];
+      if (mz > -INFINITY) acc += part_o[(row * splits + z) * dv + v] * __expf(mz - ms);
+    }
+    out[row * dv + v] = acc * inv;
+  }
+}
+
 template <typename T>
 const T* cp(const void* p) {
   return static_cast<const T*>(p);
@@ -767,13 +949,48 @@ int msgl_mix_latent_prep(const void* proj, int64_t ld_proj, float* q_abs, void* 
   return MSGL_MIX_OK;
 }
 
+int msgl_mix_latent_attn_workspace_floats(int total_q, int H, int dv, int splits) {
+  return splits > 1 ? total_q * H * splits * (dv + 2) : 0;
+}
+
 int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, const int* table, int64_t table_stride, const int* req_rows,
                          const int* seq_lens, const int* cu_q, int batch, int total_q, int H, int dk, int dv, float scale, int dtype,
-                         void* stream) {
+                         int splits, float* workspace, void* stream) {
   MIX_REQUIRE(out && q_abs && cache && table && req_rows && seq_lens && cu_q && dtype_ok(dtype), "latent_attn: null pointer / dtype");
   MIX_REQUIRE(batch >= 1 && total_q >= 0 && H >= 1 && dv >= 1 && dk >= dv, "latent_attn: bad sizes");
-  MIX_REQUIRE(dv <= 16 * kAttnMaxC, "latent_attn: value width %d above %d", dv, 16 * kAttnMaxC);
+  MIX_REQUIRE(splits >= 1 && splits <= 1024 && (splits == 1 || workspace), "latent_attn: %d splits need a workspace", splits);
   if (total_q == 0) return MSGL_MIX_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == MSGL_MIX_BF16 && dk <= 18 * 32 && dv <= 32 * 16) {
+    // matrix-core kernel: the smallest (KC, VC) instance that holds dk <= 32 KC and dv <= 16 VC (and 16 VC <= 32 KC)
+    const int HB = H < 64 ? H : 64;
+    const int QT = 64 / HB;
+    const int groups = (total_q + QT - 1) / QT + batch;
+    const dim3 grid(groups, (H + HB - 1) / HB, splits);
+    MIX_REQUIRE(grid.y <= 65535, "latent_attn: too many heads");
+    float* part_o = workspace;
+    float* part_ml = workspace ? workspace + (size_t)total_q * H * splits * dv : nullptr;
+    const int vec = (((uintptr_t)cache & 15u) == 0 && dk % 8 == 0) ? 1 : 0;
+#define ATTN_CASE(KC, VC)                                                                                                              \
+  if (dk <= KC * 32 && dv <= VC * 16) {                                                                                                \
+    hipLaunchKernelGGL((latent_attn_mfma_kernel<KC, VC>), grid, dim3(256), 0, s, out, part_o, part_ml, q_abs, cp<bf16_t>(cache), table, \
+                       table_stride, req_rows, seq_lens, cu_q, batch, H, dk, dv, scale, QT, HB, splits, vec);                          \
+    MIX_LAUNCHED("latent_attn (matrix cores)");                                                                                        \
+    if (splits > 1) {                                                                                                                  \
+      hipLaunchKernelGGL(latent_attn_merge_kernel, dim3(total_q * H), dim3(64), 0, s, out, part_o, part_ml, splits, dv);               \
+      MIX_LAUNCHED("latent_attn merge");                                                                                               \
+    }                                                                                                                                  \
+    return MSGL_MIX_OK;                                                                                                                \
+  }
+    ATTN_CASE(2, 4)
+    ATTN_CASE(4, 8)
+    ATTN_CASE(6, 8)
+    ATTN_CASE(10, 16)
+    ATTN_CASE(12, 20)
+    ATTN_CASE(18, 32)
+#undef ATTN_CASE
+  }
+  MIX_REQUIRE(dv <= 16 * kAttnMaxC, "latent_attn: value width %d above %d", dv, 16 * kAttnMaxC);
   const int HB = H < kAttnRows ? H : kAttnRows;
   const int QT = kAttnRows / HB;
   int KT = 64;
@@ -782,7 +999,6 @@ int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, cons
   const size_t lds = need(KT);
   MIX_REQUIRE(lds <= 160 * 1024, "latent_attn: key width %d does not fit LDS", dk);
   const int groups = (total_q + QT - 1) / QT + batch;  // every request may end with one partial group
-  hipStream_t s = static_cast<hipStream_t>(stream);
   DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)latent_attn_kernel<T>, lds) == 0, "latent_attn: LDS request refused");
              hipLaunchKernelGGL(latent_attn_kernel<T>, dim3(groups, (H + HB - 1) / HB), dim3(256), lds, s, out, q_abs, cp<T>(cache), table,
                                 table_stride, req_rows, seq_lens, cu_q, batch, H, dk, dv, scale, QT, HB, KT);)

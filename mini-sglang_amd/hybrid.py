@@ -284,7 +284,10 @@ class HybridDecoder:
         mixops.gemm_nt(q_abs, proj, L.uk_t, T, R, d, lda=proj.stride(0), ldb=d, ldc=H * (R + r), groups=H, a_gs=d + r,
                        b_gs=R * d, c_gs=R + r)
         o_lat = torch.empty((T, H, R), dtype=torch.float32, device=h.device)
-        mixops.latent_attn(o_lat, q_abs, rows, ctx.page_table, md.req_rows, md.seq_lens, md.cu_seqlens_q, md.batch, R, s.scale)
+        # few query rows per request (decode, short portions): cut the keys into ranges so that the launch fills the chip
+        splits = mixops.latent_attn_splits(md.batch, T, H, md.max_seqlen_k) if md.max_seqlen_q <= 16 else 1
+        mixops.latent_attn(o_lat, q_abs, rows, ctx.page_table, md.req_rows, md.seq_lens, md.cu_seqlens_q, md.batch, R, s.scale,
+                           splits=splits)
         o = torch.empty((T, H * dv), dtype=self.dtype, device=h.device)
         mixops.gemm_nt(o, o_lat, L.uv, T, dv, R, lda=H * R, ldb=R, ldc=H * dv, groups=H, a_gs=R, b_gs=dv * R, c_gs=dv)
         return mixops.linear(o, L.o)

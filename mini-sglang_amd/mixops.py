@@ -96,17 +96,29 @@ def latent_prep(proj: torch.Tensor, q_abs: torch.Tensor, cache: Optional[torch.T
         _code(proj), _stream()), "latent_prep")
 
 
+def latent_attn_splits(batch: int, total_q: int, H: int, max_keys: int) -> int:
+    """Key ranges per request for a step with few query rows: enough workgroups to fill the chip, at least 256 keys each.
+    A function of static sizes only (batch, rows, the LONGEST possible key count), so a captured graph keeps its grid."""
+    hb = min(H, 64)
+    blocks = (-(-total_q // (64 // hb)) + batch) * -(-H // hb)
+    return max(1, min(1024 // max(blocks, 1), max_keys // 256, 64))
+
+
 def latent_attn(out: torch.Tensor, q_abs: torch.Tensor, cache: torch.Tensor, table: torch.Tensor, req_rows: torch.Tensor,
-                seq_lens: torch.Tensor, cu_q: torch.Tensor, batch: int, dv: int, scale: float) -> None:
+                seq_lens: torch.Tensor, cu_q: torch.Tensor, batch: int, dv: int, scale: float, splits: int = 1) -> None:
     _dev(out, q_abs, cache, table, req_rows, seq_lens, cu_q)
     T, H, dk = q_abs.shape
     assert q_abs.dtype == torch.float32 and q_abs.is_contiguous() and out.dtype == torch.float32 and out.is_contiguous()
     assert out.shape == (T, H, dv) and cache.is_contiguous() and cache.shape[1] == dk
     assert table.dtype == torch.int32 and table.stride(1) == 1
     assert req_rows.numel() >= batch and seq_lens.numel() >= batch and cu_q.numel() >= batch + 1
+    ws = None
+    if splits > 1:
+        ws = torch.empty(mix_lib().msgl_mix_latent_attn_workspace_floats(T, H, dv, splits), dtype=torch.float32, device=out.device)
     check_mix(mix_lib().msgl_mix_latent_attn(
         out.data_ptr(), q_abs.data_ptr(), cache.data_ptr(), table.data_ptr(), table.stride(0), _i32(req_rows).data_ptr(),
-        _i32(seq_lens).data_ptr(), _i32(cu_q).data_ptr(), batch, T, H, dk, dv, float(scale), _code(cache), _stream()), "latent_attn")
+        _i32(seq_lens).data_ptr(), _i32(cu_q).data_ptr(), batch, T, H, dk, dv, float(scale), _code(cache), splits, _p(ws),
+        _stream()), "latent_attn")
 
 
 def lightning(out: torch.Tensor, qkv: torch.Tensor, state: torch.Tensor, decay: torch.Tensor, cu_q: torch.Tensor,

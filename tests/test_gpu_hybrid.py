@@ -266,29 +266,61 @@ def test_expert_products_bf16(dev):
             assert float((yh[t, k] - ref).abs().max()) < 2e-2 * float(ref.abs().max()) + 1e-3, (t, k)
 
 
-@pytest.mark.parametrize("n_keys", [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 300])
-def test_latent_attention_far_key_takes_all(dev, n_keys):
+@pytest.mark.parametrize("n_keys", [1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 300])
+@pytest.mark.parametrize("dtype,splits", [(torch.float32, 1), (torch.bfloat16, 1), (torch.bfloat16, 3)], ids=["fp32", "bf16", "bf16-split"])
+def test_latent_attention_far_key_takes_all(dev, n_keys, dtype, splits):
     """One key far back (the first, or one on a page border) is made to win the softmax for one head while another head
-    looks at the newest key: the output must be that key's latent.  Key counts sit on both sides of the kernel's key tile
-    and of the page size; the page table is shuffled."""
+    looks at the newest key: the output must be that key's latent.  Key counts sit on both sides of the kernels' key tiles
+    and of the page size; the page table is shuffled; the 16-bit cache takes the matrix-core kernel, also with the keys
+    cut into ranges that are merged afterwards (some of them empty)."""
     from mini_sglang_amd import mixops
 
     torch.manual_seed(n_keys)
     H, R, r, page = 3, 20, 6, 16
     slots = 512
-    cache = torch.randn(slots, R + r)
+    cache = torch.randn(slots, R + r).to(dtype)
     table = torch.randperm(slots)[: ((n_keys + page - 1) // page) * page].to(torch.int32).view(1, -1)
+    i32 = lambda *v: torch.tensor(v, dtype=torch.int32, device=dev)
     for far in sorted({0, min(n_keys - 1, 15), min(n_keys - 1, 16), n_keys // 2}):
         q = torch.randn(1, H, R + r) * 0.1
         cache[table[0, far]] *= 1.5
-        q[0, 0] = 40.0 * cache[table[0, far]] / cache[table[0, far]].norm()
-        q[0, 1] = 40.0 * cache[table[0, n_keys - 1]] / cache[table[0, n_keys - 1]].norm()
+        q[0, 0] = 40.0 * cache[table[0, far]].float() / cache[table[0, far]].float().norm()
+        q[0, 1] = 40.0 * cache[table[0, n_keys - 1]].float() / cache[table[0, n_keys - 1]].float().norm()
         out = torch.zeros(1, H, R, device=dev)
-        i32 = lambda *v: torch.tensor(v, dtype=torch.int32, device=dev)
-        mixops.latent_attn(out, q.to(dev), cache.to(dev), table.to(dev), i32(0), i32(n_keys), i32(0, 1), 1, R, 1.0)
+        mixops.latent_attn(out, q.to(dev), cache.to(dev), table.to(dev), i32(0), i32(n_keys), i32(0, 1), 1, R, 1.0, splits=splits)
         keys = cache[table[0, :n_keys].long()].double()
-        ref = torch.softmax(q[0].double() @ keys.T, -1) @ keys[:, :R]
-        assert torch.allclose(out[0].cpu().double(), ref, atol=2e-5)
+        qq = q[0].to(dtype).double()
+        ref = torch.softmax(qq @ keys.T, -1) @ keys[:, :R]
+        assert torch.allclose(out[0].cpu().double(), ref, atol=2e-5 if dtype == torch.float32 else 3e-2)
+
+
+def test_latent_attention_matrix_core_batch(dev):
+    """The matrix-core kernel on a mixed batch: a long portion with cached keys before it, single tokens, a short portion;
+    more heads than one 16-row tile, key and value widths off the tile sizes."""
+    from mini_sglang_amd import mixops
+
+    torch.manual_seed(11)
+    H, R, r = 20, 72, 24
+    q_lens, k_lens = [70, 1, 5, 1], [200, 333, 5, 1]
+    slots = 2048
+    cache = (torch.randn(slots, R + r) * 0.5).to(torch.bfloat16)
+    table = torch.randperm(slots)[: 4 * 352].to(torch.int32).view(4, 352)
+    T = sum(q_lens)
+    q = (torch.randn(T, H, R + r) * 0.3)
+    cu = [0]
+    for n in q_lens:
+        cu.append(cu[-1] + n)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+    out = torch.zeros(T, H, R, device=dev)
+    mixops.latent_attn(out, q.to(dev), cache.to(dev), table.to(dev), i32([0, 1, 2, 3]), i32(k_lens), i32(cu), 4, R, 0.11)
+    for b in range(4):
+        keys = cache[table[b, : k_lens[b]].long()].double()
+        for t in range(q_lens[b]):
+            pos = k_lens[b] - q_lens[b] + t
+            sc = q[cu[b] + t].to(torch.bfloat16).double() @ keys[: pos + 1].T * 0.11
+            ref = torch.softmax(sc, -1) @ keys[: pos + 1, :R]
+            got = out[cu[b] + t].cpu().double()
+            assert float((got - ref).abs().max()) < 2e-2, (b, t)
 
 
 # ----------------------------------------------------------------------------------------- schedules
