@@ -71,13 +71,14 @@ int msgl_mix_lightning(float* out, const void* qkv, int64_t ld_qkv, float* state
 int msgl_mix_gated_norm(void* out, const float* o, const void* gate, int64_t ld_gate, const void* w, float eps, int rows, int N, int dtype,
                         void* stream);
 
-/* Router: s = softmax(router h) in fp32; choice = s + bias (bias may be null); only experts of the `keep` best of G equal
- * groups of neighbours (group score = its largest choice) can win; ids = the `top` largest choices, wts = their s / (sum + 1e-20). */
-int msgl_mix_route(int* ids, float* wts, const void* h, const void* router, const void* bias, int tokens, int W, int E, int top, int G,
-                   int keep, int dtype, void* stream);
+/* Router on fp32 logits z [tokens, E] (= router weights x the token, accumulated in fp32 by a product kernel): s = softmax(z);
+ * choice = s + bias (bias in T, may be null); only experts of the `keep` best of G equal groups of neighbours (group score = its
+ * largest choice) can win; ids = the `top` largest choices, wts = their s / (sum + 1e-20). */
+int msgl_mix_route(int* ids, float* wts, const float* z, const void* bias, int tokens, int E, int top, int G, int keep, int dtype,
+                   void* stream);
 
-/* seg[E + 1], perm[n]: flat (token, choice) indices bucketed by expert, stable inside a bucket. */
-int msgl_mix_moe_sort(int* seg, int* perm, const int* ids, int n, int E, void* stream);
+/* seg[E + 1], perm[n]: flat (token, choice) indices bucketed by expert, stable inside a bucket; counts[E] is scratch. */
+int msgl_mix_moe_sort(int* seg, int* perm, int* counts, const int* ids, int n, int E, void* stream);
 
 /* C[g] = act(A[g] B[g]^T) with fp32 accumulation; groups advance by *_gs elements.  With seg, group g owns rows
  * seg[g] .. seg[g + 1] of one shared row space of at most M rows (A and C do not advance per group then); a_rows / c_rows

@@ -11,8 +11,8 @@
 //   latent_attn_kernel       one shared (c | k_r) key row for all heads, online softmax, output in latent space
 //   lightning_kernel         S <- decay * S + k v^T, o = S^T q per (request, head), state rows indexed by slot
 //   gated_norm_kernel        rms over the concatenated heads * w * sigmoid(g)
-//   route_kernel             fp32 router: softmax, bias-corrected group-limited top-k, normalised weights
-//   moe_sort_kernel          (token, choice) pairs bucketed by expert -> segment offsets + permutation
+//   route_kernel             fp32 router on fp32 logits: softmax, bias-corrected group-limited top-k, normalised weights
+//   moe_count / moe_place    (token, choice) pairs bucketed by expert -> segment offsets + permutation
 //   gemm_nt_kernel           grouped / segmented / gathered C = act(A B^T): per-head latent products, expert layers,
 //                            and every shape the library refuses
 #include <hip/hip_runtime.h>
@@ -296,15 +296,18 @@ constexpr int kLtMaxCols = 64;
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
-template <typename T>
+// R = state rows per thread (compile time): thread (column v, slice s) owns rows s R .. s R + R - 1; q and k rows are padded
+// with zeros to NS * R in LDS, so rows past d stay zero without a branch and a thread's q / k come as 16-byte LDS reads.
+template <typename T, int R>
 __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out, const T* __restrict__ qkv, int64_t ld_qkv,
                                                         float* __restrict__ state, const float* __restrict__ decay,
                                                         const int* __restrict__ cu_q, const int* __restrict__ seq_lens,
                                                         const int* __restrict__ slots, int H, int d, int dv, int CB, int NS) {
-  extern __shared__ float lds[];
-  float* sq = lds;                    // [kLtTok][d]
-  float* skk = sq + kLtTok * d;       // [kLtTok][d]
-  float* sv = skk + kLtTok * d;       // [kLtTok][CB]
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int dp = NS * R;              // padded key size
+  float* sq = lds;                    // [kLtTok][dp]
+  float* skk = sq + kLtTok * dp;      // [kLtTok][dp]
+  float* sv = skk + kLtTok * dp;      // [kLtTok][CB]
   float* part = sv + kLtTok * CB;     // [kLtTok][NS][CB]
   const int hh = blockIdx.x, b = blockIdx.y, v0 = blockIdx.z * CB;
   const int t0 = cu_q[b], n = cu_q[b + 1] - t0;
@@ -316,21 +319,21 @@ __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out,
   const bool active = s < NS && v < dv;
   float* S = state + ((size_t)slots[b] * H + hh) * d * dv;
   const float dec = decay[hh];
-  float reg[kLtMaxRows];
+  float reg[R];
 #pragma unroll
-  for (int i = 0; i < kLtMaxRows; ++i) {
-    const int row = s + i * NS;
+  for (int i = 0; i < R; ++i) {
+    const int row = s * R + i;
     reg[i] = (active && row < d && !fresh) ? S[(size_t)row * dv + v] : 0.f;
   }
   const int64_t qo = (int64_t)hh * d, ko = (int64_t)H * d + (int64_t)hh * d, vo = 2 * (int64_t)H * d + (int64_t)hh * dv + v0;
   for (int c0 = 0; c0 < n; c0 += kLtTok) {
     const int nt = min(kLtTok, n - c0);
     __syncthreads();
-    for (int e = threadIdx.x; e < nt * d; e += 256) {
-      const int tt = e / d, i = e - tt * d;
+    for (int e = threadIdx.x; e < nt * dp; e += 256) {
+      const int tt = e / dp, i = e - tt * dp;
       const T* row = qkv + (size_t)(t0 + c0 + tt) * ld_qkv;
-      sq[tt * d + i] = silu_f(ld(row + qo + i));
-      skk[tt * d + i] = silu_f(ld(row + ko + i));
+      sq[e] = i < d ? silu_f(ld(row + qo + i)) : 0.f;
+      skk[e] = i < d ? silu_f(ld(row + ko + i)) : 0.f;
     }
     for (int e = threadIdx.x; e < nt * nc; e += 256) {
       const int tt = e / nc, i = e - tt * nc;
@@ -340,14 +343,13 @@ __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out,
     if (active) {
       for (int tt = 0; tt < nt; ++tt) {
         const float vv = sv[tt * CB + vl];
+        const float* kp = skk + tt * dp + s * R;
+        const float* qp = sq + tt * dp + s * R;
         float acc = 0.f;
 #pragma unroll
-        for (int i = 0; i < kLtMaxRows; ++i) {
-          const int row = s + i * NS;
-          if (row < d) {
-            reg[i] = fmaf(dec, reg[i], skk[tt * d + row] * vv);
-            acc = fmaf(reg[i], sq[tt * d + row], acc);
-          }
+        for (int i = 0; i < R; ++i) {
+          reg[i] = fmaf(dec, reg[i], kp[i] * vv);
+          acc = fmaf(reg[i], qp[i], acc);
         }
         part[(tt * NS + s) * CB + vl] = acc;
       }
@@ -362,8 +364,8 @@ __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out,
   }
   if (active) {
 #pragma unroll
-    for (int i = 0; i < kLtMaxRows; ++i) {
-      const int row = s + i * NS;
+    for (int i = 0; i < R; ++i) {
+      const int row = s * R + i;
       if (row < d) S[(size_t)row * dv + v] = reg[i];
     }
   }
@@ -388,91 +390,118 @@ __global__ __launch_bounds__(256) void gated_norm_kernel(T* __restrict__ out, co
 }
 
 // ------------------------------------------------------------------------------------------------ router
-// One wave per token.  z = W_r h (fp32), s = softmax(z); choice = s + bias; experts outside the `keep` best groups (a group's
-// score = its largest choice) are out; the `top` largest choices win (ties: lowest index); weight = s / (sum of chosen s + 1e-20).
+// One thread per token over router logits z [T, E] that a product kernel wrote in fp32 (bf16 x bf16 products are exact in fp32,
+// so the matrix cores' fp32 accumulation IS the 32-bit router on the token's 16-bit copy).  s = softmax(z); choice = s + bias;
+// experts outside the `keep` best groups (a group's score = its largest choice) are out; the `top` largest choices win (ties:
+// lowest index); weight = s / (sum of chosen s + 1e-20).  Scores live in LDS columns, one per thread.
 template <typename T>
-__global__ __launch_bounds__(64) void route_kernel(int* __restrict__ ids, float* __restrict__ wts, const T* __restrict__ h,
-                                                   const T* __restrict__ router, const T* __restrict__ bias, int E, int top, int G,
-                                                   int keep, int W) {
+__global__ __launch_bounds__(64) void route_kernel(int* __restrict__ ids, float* __restrict__ wts, const float* __restrict__ z,
+                                                   const T* __restrict__ bias, int tokens, int E, int top, int G, int keep, int TPB) {
   extern __shared__ float lds[];
-  float* s = lds;           // [E] softmax scores
-  float* c = s + E;         // [E] choice scores
-  float* gs = c + E;        // [G]
-  const int t = blockIdx.x, lane = threadIdx.x;
-  const T* x = h + (size_t)t * W;
+  const int t = blockIdx.x * TPB + threadIdx.x;
+  if (threadIdx.x >= TPB || t >= tokens) return;
+  float* s = lds + threadIdx.x;             // s[e * TPB]
+  float* c = lds + (size_t)E * TPB + threadIdx.x;
+  const float* zr = z + (size_t)t * E;
+  float mx = -INFINITY;
+  for (int e = 0; e < E; ++e) mx = fmaxf(mx, zr[e]);
+  float sum = 0.f;
   for (int e = 0; e < E; ++e) {
-    float acc = 0.f;
-    for (int i = lane; i < W; i += 64) acc = fmaf(ld(x + i), ld(router + (size_t)e * W + i), acc);
-    acc = wave_sum(acc);
-    if (lane == 0) s[e] = acc;
+    const float v = expf(zr[e] - mx);
+    s[e * TPB] = v;
+    sum += v;
   }
-  __syncthreads();
-  if (lane == 0) {
-    float mx = -INFINITY;
-    for (int e = 0; e < E; ++e) mx = fmaxf(mx, s[e]);
-    float sum = 0.f;
-    for (int e = 0; e < E; ++e) {
-      s[e] = expf(s[e] - mx);
-      sum += s[e];
-    }
-    for (int e = 0; e < E; ++e) {
-      s[e] /= sum;
-      c[e] = s[e] + (bias ? ld(bias + e) : 0.f);
-    }
-    const int per = E / G;
-    if (keep < G) {
-      for (int g = 0; g < G; ++g) {
-        float b = -INFINITY;
-        for (int e = g * per; e < (g + 1) * per; ++e) b = fmaxf(b, c[e]);
-        gs[g] = b;
-      }
-      // a group stays if fewer than `keep` groups beat it (ties: the lower index wins)
-      for (int g = 0; g < G; ++g) {
-        int better = 0;
-        for (int o2 = 0; o2 < G; ++o2) better += (gs[o2] > gs[g]) || (gs[o2] == gs[g] && o2 < g);
-        if (better >= keep)
-          for (int e = g * per; e < (g + 1) * per; ++e) c[e] = -INFINITY;
-      }
-    }
-    float tot = 0.f;
-    for (int k = 0; k < top; ++k) {
-      int best = -1;
-      float bv = -INFINITY;
-      for (int e = 0; e < E; ++e)
-        if (c[e] > bv) {
-          best = e;
-          bv = c[e];
-        }
-      if (best < 0) best = 0;  // unreachable: the host checks top <= keep * (E / G) and choice scores are finite
-      ids[(size_t)t * top + k] = best;
-      wts[(size_t)t * top + k] = s[best];
-      tot += s[best];
-      c[best] = -INFINITY;
-    }
-    for (int k = 0; k < top; ++k) wts[(size_t)t * top + k] /= (tot + 1e-20f);
+  for (int e = 0; e < E; ++e) {
+    const float v = s[e * TPB] / sum;
+    s[e * TPB] = v;
+    c[e * TPB] = v + (bias ? ld(bias + e) : 0.f);
   }
+  const int per = E / G;
+  if (keep < G) {
+    // a group stays if fewer than `keep` groups beat it (ties: the lower index wins)
+    for (int g = 0; g < G; ++g) {
+      float mine = -INFINITY;
+      for (int e = g * per; e < (g + 1) * per; ++e) mine = fmaxf(mine, s[e * TPB] + (bias ? ld(bias + e) : 0.f));
+      int better = 0;
+      for (int o2 = 0; o2 < G; ++o2) {
+        if (o2 == g) continue;
+        float other = -INFINITY;
+        for (int e = o2 * per; e < (o2 + 1) * per; ++e) other = fmaxf(other, s[e * TPB] + (bias ? ld(bias + e) : 0.f));
+        better += (other > mine) || (other == mine && o2 < g);
+      }
+      if (better >= keep)
+        for (int e = g * per; e < (g + 1) * per; ++e) c[e * TPB] = -INFINITY;
+    }
+  }
+  float tot = 0.f;
+  for (int k = 0; k < top; ++k) {
+    int best = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      const float v = c[e * TPB];
+      if (v > bv) {
+        best = e;
+        bv = v;
+      }
+    }
+    if (best < 0) best = 0;  // unreachable: the host checks top <= keep * (E / G) and choice scores are finite
+    ids[(size_t)t * top + k] = best;
+    const float sv = s[best * TPB];
+    wts[(size_t)t * top + k] = sv;
+    tot += sv;
+    c[best * TPB] = -INFINITY;
+  }
+  for (int k = 0; k < top; ++k) wts[(size_t)t * top + k] /= (tot + 1e-20f);
 }
 
 // ------------------------------------------------------------------------------------------------ expert bucketing
-// One workgroup.  seg[e] .. seg[e + 1] = the sorted positions of expert e; perm[position] = flat (token * top + choice).
-// Positions inside a segment follow the flat index (stable), so the layout does not depend on scheduling.
-__global__ __launch_bounds__(256) void moe_sort_kernel(int* __restrict__ seg, int* __restrict__ perm, const int* __restrict__ ids, int n,
-                                                       int E) {
-  extern __shared__ int li[];  // [E + 1]
-  for (int e = threadIdx.x; e <= E; e += 256) li[e] = 0;
+// seg[e] .. seg[e + 1] = the sorted positions of expert e; perm[position] = flat (token * top + choice), in flat order inside a
+// segment (stable: the layout does not depend on scheduling).  Two launches of one workgroup per expert, no atomics and nothing
+// to clear: first every expert counts its entries, then it adds up the counts before it and places its entries by a running
+// workgroup-wide rank.
+__device__ __forceinline__ int block_rank256(bool flag, int* wsum, int& total) {
+  const unsigned long long bal = __ballot(flag);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int before = __popcll(bal & ((1ull << lane) - 1ull));
   __syncthreads();
-  for (int i = threadIdx.x; i < n; i += 256) atomicAdd(&li[ids[i] + 1], 1);
+  if (lane == 0) wsum[wave] = __popcll(bal);
   __syncthreads();
-  if (threadIdx.x == 0) {
-    for (int e = 0; e < E; ++e) li[e + 1] += li[e];
+  int off = 0;
+  for (int w = 0; w < wave; ++w) off += wsum[w];
+  total = wsum[0] + wsum[1] + wsum[2] + wsum[3];
+  return off + before;
+}
+
+__global__ __launch_bounds__(256) void moe_count_kernel(int* __restrict__ counts, const int* __restrict__ ids, int n) {
+  __shared__ int wsum[4];
+  const int e = blockIdx.x;
+  int cnt = 0;
+  for (int i0 = 0; i0 < n; i0 += 256) {
+    const int i = i0 + threadIdx.x;
+    int tot;
+    block_rank256(i < n && ids[i] == e, wsum, tot);
+    cnt += tot;
   }
-  __syncthreads();
-  for (int e = threadIdx.x; e <= E; e += 256) seg[e] = li[e];
-  // stable placement: thread e walks the flat list for its expert
-  for (int e = threadIdx.x; e < E; e += 256) {
-    int p = li[e];
-    for (int i = 0; i < n; ++i)
-      if (ids[i] == e) perm[p++] = i;
+  if (threadIdx.x == 0) counts[e] = cnt;
+}
+
+__global__ __launch_bounds__(256) void moe_place_kernel(int* __restrict__ seg, int* __restrict__ perm, const int* __restrict__ counts,
+                                                        const int* __restrict__ ids, int n, int E) {
+  __shared__ int wsum[4];
+  const int e = blockIdx.x;
+  int base = 0;
+  for (int k = 0; k < e; ++k) base += counts[k];
+  if (threadIdx.x == 0) {
+    seg[e] = base;
+    if (e == E - 1) seg[E] = base + counts[e];
+  }
+  for (int i0 = 0; i0 < n; i0 += 256) {
+    const int i = i0 + threadIdx.x;
+    const bool mine = i < n && ids[i] == e;
+    int tot;
+    const int rank = block_rank256(mine, wsum, tot);
+    if (mine) perm[base + rank] = i;
+    base += tot;
   }
 }
 
@@ -1013,16 +1042,28 @@ int msgl_mix_lightning(float* out, const void* qkv, int64_t ld_qkv, float* state
   MIX_REQUIRE(ld_qkv >= (int64_t)H * (2 * d + dv), "lightning: projection row too short");
   const int CB = dv < kLtMaxCols ? dv : kLtMaxCols;
   const int NS = 256 / CB;
-  MIX_REQUIRE((d + NS - 1) / NS <= kLtMaxRows, "lightning: key size %d needs more than %d state rows per thread", d, kLtMaxRows);
+  const int need = (d + NS - 1) / NS;
+  MIX_REQUIRE(need <= kLtMaxRows, "lightning: key size %d needs more than %d state rows per thread", d, kLtMaxRows);
   const int col_blocks = (dv + CB - 1) / CB;
   MIX_REQUIRE(col_blocks <= 65535, "lightning: value width %d", dv);
-  const size_t lds = (size_t)(kLtTok * (2 * d + CB) + kLtTok * NS * CB) * sizeof(float);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)lightning_kernel<T>, lds) == 0, "lightning: LDS request refused");
-             hipLaunchKernelGGL(lightning_kernel<T>, dim3(H, batch, col_blocks), dim3(256), lds, s, out, cp<T>(qkv), ld_qkv, state, decay,
-                                cu_q, seq_lens, slots, H, d, dv, CB, NS);)
-  MIX_LAUNCHED("lightning");
-  return MSGL_MIX_OK;
+  const dim3 grid(H, batch, col_blocks);
+#define LT_CASE(RR)                                                                                                                    \
+  if (need <= RR) {                                                                                                                    \
+    const size_t lds = (size_t)(kLtTok * (2 * NS * RR + CB) + kLtTok * NS * CB) * sizeof(float);                                       \
+    DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)lightning_kernel<T, RR>, lds) == 0, "lightning: LDS request refused");       \
+               hipLaunchKernelGGL((lightning_kernel<T, RR>), grid, dim3(256), lds, s, out, cp<T>(qkv), ld_qkv, state, decay, cu_q,     \
+                                  seq_lens, slots, H, d, dv, CB, NS);)                                                                 \
+    MIX_LAUNCHED("lightning");                                                                                                         \
+    return MSGL_MIX_OK;                                                                                                                \
+  }
+  LT_CASE(4)
+  LT_CASE(8)
+  LT_CASE(16)
+  LT_CASE(32)
+  LT_CASE(64)
+#undef LT_CASE
+  return MSGL_MIX_EINVAL;
 }
 
 int msgl_mix_gated_norm(void* out, const float* o, const void* gate, int64_t ld_gate, const void* w, float eps, int rows, int N, int dtype,
@@ -1035,26 +1076,30 @@ int msgl_mix_gated_norm(void* out, const float* o, const void* gate, int64_t ld_
   return MSGL_MIX_OK;
 }
 
-int msgl_mix_route(int* ids, float* wts, const void* h, const void* router, const void* bias, int tokens, int W, int E, int top, int G,
-                   int keep, int dtype, void* stream) {
-  MIX_REQUIRE(ids && wts && h && router && dtype_ok(dtype), "route: null pointer / dtype");
+int msgl_mix_route(int* ids, float* wts, const float* z, const void* bias, int tokens, int E, int top, int G, int keep, int dtype,
+                   void* stream) {
+  MIX_REQUIRE(ids && wts && z && dtype_ok(dtype), "route: null pointer / dtype");
   MIX_REQUIRE(E >= 1 && top >= 1 && top <= E && G >= 1 && E % G == 0 && keep >= 1 && keep <= G && top <= keep * (E / G),
               "route: bad sizes E %d top %d groups %d keep %d", E, top, G, keep);
   if (tokens == 0) return MSGL_MIX_OK;
-  const size_t lds = (size_t)(2 * E + G) * sizeof(float);
+  int tpb = 64;
+  while (tpb > 1 && (size_t)2 * E * tpb * sizeof(float) > 64 * 1024) tpb >>= 1;
+  const size_t lds = (size_t)2 * E * tpb * sizeof(float);
   MIX_REQUIRE(lds <= 64 * 1024, "route: too many experts");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  DISPATCH_T(dtype, hipLaunchKernelGGL(route_kernel<T>, dim3(tokens), dim3(64), lds, s, ids, wts, cp<T>(h), cp<T>(router), cp<T>(bias), E, top,
-                                       G, keep, W);)
+  DISPATCH_T(dtype, hipLaunchKernelGGL(route_kernel<T>, dim3((tokens + tpb - 1) / tpb), dim3(64), lds, s, ids, wts, z, cp<T>(bias), tokens, E,
+                                       top, G, keep, tpb);)
   MIX_LAUNCHED("route");
   return MSGL_MIX_OK;
 }
 
-int msgl_mix_moe_sort(int* seg, int* perm, const int* ids, int n, int E, void* stream) {
-  MIX_REQUIRE(seg && perm && ids && n >= 0 && E >= 1 && E <= 8192, "moe_sort: bad arguments");
+int msgl_mix_moe_sort(int* seg, int* perm, int* counts, const int* ids, int n, int E, void* stream) {
+  MIX_REQUIRE(seg && perm && counts && ids && n >= 0 && E >= 1 && E <= 65535, "moe_sort: bad arguments");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(256), (size_t)(E + 1) * sizeof(int), s, seg, perm, ids, n, E);
-  MIX_LAUNCHED("moe_sort");
+  hipLaunchKernelGGL(moe_count_kernel, dim3(E), dim3(256), 0, s, counts, ids, n);
+  MIX_LAUNCHED("moe_sort (count)");
+  hipLaunchKernelGGL(moe_place_kernel, dim3(E), dim3(256), 0, s, seg, perm, counts, ids, n, E);
+  MIX_LAUNCHED("moe_sort (place)");
   return MSGL_MIX_OK;
 }
 

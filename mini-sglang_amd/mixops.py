@@ -145,16 +145,19 @@ def gated_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: f
 
 
 def route(h: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int, groups: int, keep: int):
-    """-> (expert ids int32 [T, top], weights fp32 [T, top])."""
+    """-> (expert ids int32 [T, top], weights fp32 [T, top]).  Router logits in fp32 (fp32 accumulation over the token's copy in
+    the model dtype: 16-bit products are exact in fp32), then softmax, corrected group-limited choice and weights in one pass."""
     _dev(h, router, bias)
     T, W = h.shape
     E = router.shape[0]
     assert h.is_contiguous() and router.is_contiguous() and router.shape == (E, W) and router.dtype == h.dtype
     assert bias is None or (bias.dtype == h.dtype and bias.shape == (E,) and bias.is_contiguous())
+    z = torch.empty((T, E), dtype=torch.float32, device=h.device)
+    gemm_nt(z, h, router, T, E, W, lda=W, ldb=W, ldc=E)
     ids = torch.empty((T, top), dtype=torch.int32, device=h.device)
     wts = torch.empty((T, top), dtype=torch.float32, device=h.device)
-    check_mix(mix_lib().msgl_mix_route(ids.data_ptr(), wts.data_ptr(), h.data_ptr(), router.data_ptr(), _p(bias), T, W, E, top,
-                                       groups, keep, _code(h), _stream()), "route")
+    check_mix(mix_lib().msgl_mix_route(ids.data_ptr(), wts.data_ptr(), z.data_ptr(), _p(bias), T, E, top, groups, keep, _code(h),
+                                       _stream()), "route")
     return ids, wts
 
 
@@ -162,10 +165,11 @@ def moe_sort(ids: torch.Tensor, experts: int):
     """-> (segment offsets int32 [E + 1], permutation int32 [T * top])."""
     _dev(ids)
     n = ids.numel()
-    seg = torch.empty(experts + 1, dtype=torch.int32, device=ids.device)
+    seg = torch.empty(2 * experts + 1, dtype=torch.int32, device=ids.device)  # offsets, then the per-expert counts (scratch)
     perm = torch.empty(max(n, 1), dtype=torch.int32, device=ids.device)
-    check_mix(mix_lib().msgl_mix_moe_sort(seg.data_ptr(), perm.data_ptr(), _i32(ids).data_ptr(), n, experts, _stream()), "moe_sort")
-    return seg, perm
+    check_mix(mix_lib().msgl_mix_moe_sort(seg.data_ptr(), perm.data_ptr(), seg[experts + 1:].data_ptr(), _i32(ids).data_ptr(), n,
+                                          experts, _stream()), "moe_sort")
+    return seg[: experts + 1], perm
 
 
 def gemm_nt(C: torch.Tensor, A: torch.Tensor, B: torch.Tensor, M: int, N: int, K: int, *, lda: int, ldb: int, ldc: int,

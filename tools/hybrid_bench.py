@@ -133,7 +133,8 @@ def kernel_rooflines(name: str, prompt: int, batch: int, device) -> dict:
         # --- latent attention over the shared latent rows
         cache, q_abs = rnd(slots, R + r), rnd(T, H, R + r, dtype=torch.float32, scale=0.1)
         o_lat = torch.empty(T, H, R, dtype=torch.float32, device=device)
-        us = _time_us(lambda: mixops.latent_attn(o_lat, q_abs, cache, table, rows, seq, cu, reqs, R, 0.1))
+        splits = mixops.latent_attn_splits(reqs, T, H, ctx) if q_len <= 16 else 1
+        us = _time_us(lambda: mixops.latent_attn(o_lat, q_abs, cache, table, rows, seq, cu, reqs, R, 0.1, splits=splits))
         pairs = reqs * (q_len * (ctx - q_len) + q_len * (q_len + 1) // 2)
         flops = 2.0 * pairs * H * (2 * R + r)
         byts = reqs * ctx * (R + r) * 2 + T * H * (2 * R + r) * 4
