@@ -63,9 +63,14 @@ int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, cons
 
 /* Linear recurrence per (request, head): S <- decay[h] S + k v^T, out = S^T q, with q, k, v = SiLU of the projection row
  * [q: H x d | k: H x d | v: H x dv | ...].  state: fp32 [slots, H, d, dv], row slots[b]; a request whose first new token is at
- * position 0 (seq_lens[b] == its new tokens) starts from zero.  out: fp32 [tokens, H * dv]. */
+ * position 0 (seq_lens[b] == its new tokens) starts from zero.  out: fp32 [tokens, H * dv].
+ * n_items > 0: the new tokens are cut into chunks that run in parallel -- items[3 i] = (request, first token, end token) with
+ * offsets from the request's first new token, every request's chunks in order and covering all its new tokens, item_first[b] ..
+ * item_first[b + 1] = the chunks of request b; three launches (every chunk's own state contribution, a scan over the chunks
+ * of a request, every chunk's outputs from the state before it); scratch: fp32 [n_items, H, d, dv]. */
 int msgl_mix_lightning(float* out, const void* qkv, int64_t ld_qkv, float* state, const float* decay, const int* cu_q, const int* seq_lens,
-                       const int* slots, int batch, int H, int d, int dv, int dtype, void* stream);
+                       const int* slots, int batch, int H, int d, int dv, int dtype, int n_items, const int* items, const int* item_first,
+                       float* scratch, void* stream);
 
 /* out = o / sqrt(mean(o^2) + eps) * w * sigmoid(gate) over rows of N (o fp32, out and gate T). */
 int msgl_mix_gated_norm(void* out, const float* o, const void* gate, int64_t ld_gate, const void* w, float eps, int rows, int N, int dtype,

@@ -148,7 +148,7 @@ MIX_SIGNATURES = {
     "msgl_mix_latent_prep": (_i, [_p, _l, _p, _p, _p, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "msgl_mix_latent_attn_workspace_floats": (_i, [_i, _i, _i, _i]),
     "msgl_mix_latent_attn": (_i, [_p, _p, _p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p, _p]),
-    "msgl_mix_lightning": (_i, [_p, _p, _l, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_lightning": (_i, [_p, _p, _l, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
     "msgl_mix_gated_norm": (_i, [_p, _p, _p, _l, _p, _f, _i, _i, _i, _p]),
     "msgl_mix_route": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "msgl_mix_moe_sort": (_i, [_p, _p, _p, _p, _i, _i, _p]),

@@ -35,6 +35,7 @@ class HipAttnMetadata:
     total_tiles: int = 0
     tile_order: Optional[torch.Tensor] = None  # [total_tiles] int32: q tiles, most keys first (prefill only)
     plan: Optional[torch.Tensor] = None     # decode work list (device)
+    chunks: Optional[tuple] = None          # recurrent layers: (items [n, 3], item_first [B + 1], n) of long portions cut in pieces
 
     def get_last_indices(self, bs: int) -> torch.Tensor:
         return self.cu_seqlens_q[1: 1 + bs] - 1
@@ -220,6 +221,8 @@ class MixAttnBackend:
     the two in one launch, so there is no prefill / decode split and no work plan; the recurrent layers use the table row
     as the request's state slot.  Graph capture keeps static copies of the vectors, refreshed before every replay."""
 
+    RECURRENT_CHUNK = 128
+
     def __init__(self, config: Any, ctx: Any = None, *, tp_size: int = 1) -> None:
         ctx = ctx if ctx is not None else _core.get_global_ctx()
         self.ctx, self.config = ctx, config
@@ -235,13 +238,26 @@ class MixAttnBackend:
         q = np.fromiter((r.extend_len for r in reqs), dtype=np.int64, count=bs)
         k = np.fromiter((r.device_len for r in reqs), dtype=np.int64, count=bs)
         rows = np.fromiter((r.table_idx for r in reqs), dtype=np.int64, count=bs)
-        host = torch.empty(3 * bs + 1, dtype=torch.int32, pin_memory=True)
+        # a long portion's recurrence runs as pieces of RECURRENT_CHUNK tokens in parallel (their states joined by a scan)
+        pieces = -(-q // self.RECURRENT_CHUNK)
+        n_items = int(pieces.sum()) if int(q.max()) >= 2 * self.RECURRENT_CHUNK else 0
+        host = torch.empty(3 * bs + 1 + (3 * n_items + bs + 1 if n_items else 0), dtype=torch.int32, pin_memory=True)
         h = host.numpy()
         h[:bs], h[bs: 2 * bs], h[2 * bs] = k, rows, 0
-        h[2 * bs + 1:] = np.cumsum(q)
+        h[2 * bs + 1: 3 * bs + 1] = np.cumsum(q)
+        if n_items:
+            req = np.repeat(np.arange(bs), pieces)
+            first = np.cumsum(pieces) - pieces
+            begin = (np.arange(n_items) - first[req]) * self.RECURRENT_CHUNK
+            items = h[3 * bs + 1: 3 * bs + 1 + 3 * n_items].reshape(n_items, 3)
+            items[:, 0], items[:, 1], items[:, 2] = req, begin, np.minimum(begin + self.RECURRENT_CHUNK, q[req])
+            h[3 * bs + 1 + 3 * n_items] = 0
+            h[3 * bs + 2 + 3 * n_items:] = np.cumsum(pieces)
         dev = host.to(self.device, non_blocking=True)
-        batch.attn_metadata = HipAttnMetadata(cu_seqlens_q=dev[2 * bs:], seq_lens=dev[:bs], req_rows=dev[bs: 2 * bs], batch=bs,
+        batch.attn_metadata = HipAttnMetadata(cu_seqlens_q=dev[2 * bs: 3 * bs + 1], seq_lens=dev[:bs], req_rows=dev[bs: 2 * bs], batch=bs,
                                               max_seqlen_q=int(q.max()), max_seqlen_k=int(k.max()))
+        if n_items:
+            batch.attn_metadata.chunks = (dev[3 * bs + 1: 3 * bs + 1 + 3 * n_items], dev[3 * bs + 1 + 3 * n_items:], n_items)
 
     # ------------------------------------------------------------------ graph hooks
     def init_capture_graph(self, max_seq_len: int, bs_list: List[int]) -> None:

@@ -302,22 +302,33 @@ template <typename T, int R>
 __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out, const T* __restrict__ qkv, int64_t ld_qkv,
                                                         float* __restrict__ state, const float* __restrict__ decay,
                                                         const int* __restrict__ cu_q, const int* __restrict__ seq_lens,
-                                                        const int* __restrict__ slots, int H, int d, int dv, int CB, int NS) {
+                                                        const int* __restrict__ slots, int H, int d, int dv, int CB, int NS,
+                                                        const int* __restrict__ items, float* __restrict__ scratch, int mode) {
+  // mode 0: one workgroup row per request, state row in and out.  With `items` (request, first token, end token of a chunk of a
+  // long portion; offsets from the request's first new token): mode 1 = the chunk's own contribution to the state from zero
+  // -> scratch[item], no outputs; mode 2 = outputs of the chunk from the state before it (scratch[item], written by the scan).
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int dp = NS * R;              // padded key size
   float* sq = lds;                    // [kLtTok][dp]
   float* skk = sq + kLtTok * dp;      // [kLtTok][dp]
   float* sv = skk + kLtTok * dp;      // [kLtTok][CB]
   float* part = sv + kLtTok * CB;     // [kLtTok][NS][CB]
-  const int hh = blockIdx.x, b = blockIdx.y, v0 = blockIdx.z * CB;
-  const int t0 = cu_q[b], n = cu_q[b + 1] - t0;
+  const int hh = blockIdx.x, v0 = blockIdx.z * CB;
+  const int b = mode ? items[3 * blockIdx.y] : blockIdx.y;
+  int t0 = cu_q[b], n = cu_q[b + 1] - t0;
   if (n <= 0) return;
-  const bool fresh = seq_lens[b] - n == 0;
+  bool fresh = seq_lens[b] - n == 0;
+  float* S = state + ((size_t)slots[b] * H + hh) * d * dv;
+  if (mode) {
+    t0 += items[3 * blockIdx.y + 1];
+    n = items[3 * blockIdx.y + 2] - items[3 * blockIdx.y + 1];
+    fresh = mode == 1;
+    S = scratch + ((size_t)blockIdx.y * H + hh) * d * dv;
+  }
   const int vl = threadIdx.x % CB, s = threadIdx.x / CB;
   const int v = v0 + vl;
   const int nc = min(CB, dv - v0);  // columns of this block
   const bool active = s < NS && v < dv;
-  float* S = state + ((size_t)slots[b] * H + hh) * d * dv;
   const float dec = decay[hh];
   float reg[R];
 #pragma unroll
@@ -332,7 +343,7 @@ __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out,
     for (int e = threadIdx.x; e < nt * dp; e += 256) {
       const int tt = e / dp, i = e - tt * dp;
       const T* row = qkv + (size_t)(t0 + c0 + tt) * ld_qkv;
-      sq[e] = i < d ? silu_f(ld(row + qo + i)) : 0.f;
+      if (mode != 1) sq[e] = i < d ? silu_f(ld(row + qo + i)) : 0.f;
       skk[e] = i < d ? silu_f(ld(row + ko + i)) : 0.f;
     }
     for (int e = threadIdx.x; e < nt * nc; e += 256) {
@@ -340,7 +351,14 @@ __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out,
       sv[tt * CB + i] = silu_f(ld(qkv + (size_t)(t0 + c0 + tt) * ld_qkv + vo + i));
     }
     __syncthreads();
-    if (active) {
+    if (active && mode == 1) {
+      for (int tt = 0; tt < nt; ++tt) {
+        const float vv = sv[tt * CB + vl];
+        const float* kp = skk + tt * dp + s * R;
+#pragma unroll
+        for (int i = 0; i < R; ++i) reg[i] = fmaf(dec, reg[i], kp[i] * vv);
+      }
+    } else if (active) {
       for (int tt = 0; tt < nt; ++tt) {
         const float vv = sv[tt * CB + vl];
         const float* kp = skk + tt * dp + s * R;
@@ -354,6 +372,7 @@ __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out,
         part[(tt * NS + s) * CB + vl] = acc;
       }
     }
+    if (mode == 1) continue;
     __syncthreads();
     for (int e = threadIdx.x; e < nt * nc; e += 256) {
       const int tt = e / nc, i = e - tt * nc;
@@ -362,13 +381,37 @@ __global__ __launch_bounds__(256) void lightning_kernel(float* __restrict__ out,
       out[(size_t)(t0 + c0 + tt) * ((size_t)H * dv) + (size_t)hh * dv + v0 + i] = acc;
     }
   }
-  if (active) {
+  if (active && mode != 2) {
 #pragma unroll
     for (int i = 0; i < R; ++i) {
       const int row = s * R + i;
       if (row < d) S[(size_t)row * dv + v] = reg[i];
     }
   }
+}
+
+// Between the two chunk passes: per state element, walk a request's chunks in order.  scratch[item] holds the chunk's own
+// contribution U on entry and the state BEFORE the chunk on exit; S <- decay^len S + U; the state row gets the last S.
+__global__ __launch_bounds__(256) void lightning_scan_kernel(float* __restrict__ state, float* __restrict__ scratch,
+                                                             const float* __restrict__ decay, const int* __restrict__ cu_q,
+                                                             const int* __restrict__ seq_lens, const int* __restrict__ slots,
+                                                             const int* __restrict__ items, const int* __restrict__ item_first, int H,
+                                                             int dd) {
+  const int hh = blockIdx.x, b = blockIdx.y;
+  const int e = blockIdx.z * 256 + threadIdx.x;
+  const int i0 = item_first[b], i1 = item_first[b + 1];
+  if (e >= dd || i0 >= i1) return;
+  const int n = cu_q[b + 1] - cu_q[b];
+  float* S = state + ((size_t)slots[b] * H + hh) * dd + e;
+  float cur = (seq_lens[b] - n == 0) ? 0.f : *S;
+  const float lg = logf(decay[hh]);
+  for (int i = i0; i < i1; ++i) {
+    float* u = scratch + ((size_t)i * H + hh) * dd + e;
+    const float add = *u;
+    *u = cur;
+    cur = fmaf(expf((float)(items[3 * i + 2] - items[3 * i + 1]) * lg), cur, add);
+  }
+  *S = cur;
 }
 
 // ------------------------------------------------------------------------------------------------ gated norm
@@ -1036,10 +1079,12 @@ int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, cons
 }
 
 int msgl_mix_lightning(float* out, const void* qkv, int64_t ld_qkv, float* state, const float* decay, const int* cu_q, const int* seq_lens,
-                       const int* slots, int batch, int H, int d, int dv, int dtype, void* stream) {
+                       const int* slots, int batch, int H, int d, int dv, int dtype, int n_items, const int* items, const int* item_first,
+                       float* scratch, void* stream) {
   MIX_REQUIRE(out && qkv && state && decay && cu_q && seq_lens && slots && dtype_ok(dtype), "lightning: null pointer / dtype");
   MIX_REQUIRE(batch >= 1 && batch <= 65535 && H >= 1 && d >= 1 && dv >= 1, "lightning: bad sizes");
   MIX_REQUIRE(ld_qkv >= (int64_t)H * (2 * d + dv), "lightning: projection row too short");
+  MIX_REQUIRE(n_items == 0 || (items && item_first && scratch && n_items <= 65535), "lightning: chunk list without its arrays");
   const int CB = dv < kLtMaxCols ? dv : kLtMaxCols;
   const int NS = 256 / CB;
   const int need = (d + NS - 1) / NS;
@@ -1047,14 +1092,21 @@ int msgl_mix_lightning(float* out, const void* qkv, int64_t ld_qkv, float* state
   const int col_blocks = (dv + CB - 1) / CB;
   MIX_REQUIRE(col_blocks <= 65535, "lightning: value width %d", dv);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(H, batch, col_blocks);
+#define LT_LAUNCH(RR, ROWS, MODE)                                                                                                      \
+  hipLaunchKernelGGL((lightning_kernel<T, RR>), dim3(H, ROWS, col_blocks), dim3(256), lds, s, out, cp<T>(qkv), ld_qkv, state, decay,   \
+                     cu_q, seq_lens, slots, H, d, dv, CB, NS, items, scratch, MODE);                                                   \
+  MIX_LAUNCHED("lightning");
 #define LT_CASE(RR)                                                                                                                    \
   if (need <= RR) {                                                                                                                    \
     const size_t lds = (size_t)(kLtTok * (2 * NS * RR + CB) + kLtTok * NS * CB) * sizeof(float);                                       \
     DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)lightning_kernel<T, RR>, lds) == 0, "lightning: LDS request refused");       \
-               hipLaunchKernelGGL((lightning_kernel<T, RR>), grid, dim3(256), lds, s, out, cp<T>(qkv), ld_qkv, state, decay, cu_q,     \
-                                  seq_lens, slots, H, d, dv, CB, NS);)                                                                 \
-    MIX_LAUNCHED("lightning");                                                                                                         \
+               if (n_items == 0) { LT_LAUNCH(RR, batch, 0) } else {                                                                    \
+                 LT_LAUNCH(RR, n_items, 1)                                                                                             \
+                 hipLaunchKernelGGL(lightning_scan_kernel, dim3(H, batch, (d * dv + 255) / 256), dim3(256), 0, s, state, scratch,      \
+                                    decay, cu_q, seq_lens, slots, items, item_first, H, d * dv);                                       \
+                 MIX_LAUNCHED("lightning scan");                                                                                       \
+                 LT_LAUNCH(RR, n_items, 2)                                                                                             \
+               })                                                                                                                      \
     return MSGL_MIX_OK;                                                                                                                \
   }
   LT_CASE(4)
@@ -1063,6 +1115,7 @@ int msgl_mix_lightning(float* out, const void* qkv, int64_t ld_qkv, float* state
   LT_CASE(32)
   LT_CASE(64)
 #undef LT_CASE
+#undef LT_LAUNCH
   return MSGL_MIX_EINVAL;
 }
 

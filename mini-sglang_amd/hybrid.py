@@ -297,7 +297,8 @@ class HybridDecoder:
         T, H, d, dv = h.shape[0], s.heads, s.dim, s.vdim
         proj = mixops.linear(h, L.w_in)
         o = torch.empty((T, H * dv), dtype=torch.float32, device=h.device)
-        mixops.lightning(o, proj, ctx.kv_cache.state(i), L.decay, md.cu_seqlens_q, md.seq_lens, md.req_rows, md.batch)
+        mixops.lightning(o, proj, ctx.kv_cache.state(i), L.decay, md.cu_seqlens_q, md.seq_lens, md.req_rows, md.batch,
+                         chunks=getattr(md, "chunks", None))
         gated = mixops.gated_norm(o, proj[:, 2 * H * d + H * dv:], L.out_norm, self.cfg.rms_norm_eps)
         return mixops.linear(gated, L.o)
 

@@ -122,15 +122,24 @@ def latent_attn(out: torch.Tensor, q_abs: torch.Tensor, cache: torch.Tensor, tab
 
 
 def lightning(out: torch.Tensor, qkv: torch.Tensor, state: torch.Tensor, decay: torch.Tensor, cu_q: torch.Tensor,
-              seq_lens: torch.Tensor, slots: torch.Tensor, batch: int) -> None:
-    """state: fp32 [slots, H, d, dv]; qkv rows = [q H*d | k H*d | v H*dv | anything]."""
+              seq_lens: torch.Tensor, slots: torch.Tensor, batch: int, chunks=None) -> None:
+    """state: fp32 [slots, H, d, dv]; qkv rows = [q H*d | k H*d | v H*dv | anything].  chunks = (items int32 [n, 3], item_first
+    int32 [batch + 1], n) cuts long portions into pieces that run in parallel (see include/msgl_mix.h)."""
     _dev(out, qkv, state, decay, cu_q, seq_lens, slots)
     _, H, d, dv = state.shape
     assert state.dtype == torch.float32 and state.is_contiguous() and decay.dtype == torch.float32 and decay.shape == (H,)
     assert out.dtype == torch.float32 and out.is_contiguous() and out.shape == (qkv.shape[0], H * dv) and qkv.stride(1) == 1
+    items = first = scratch = None
+    n_items = 0
+    if chunks is not None:
+        items, first, n_items = chunks
+        _dev(items, first)
+        assert items.numel() == 3 * n_items and first.numel() == batch + 1
+        scratch = torch.empty((n_items, H, d, dv), dtype=torch.float32, device=out.device)
     check_mix(mix_lib().msgl_mix_lightning(
         out.data_ptr(), qkv.data_ptr(), qkv.stride(0), state.data_ptr(), decay.data_ptr(), _i32(cu_q).data_ptr(),
-        _i32(seq_lens).data_ptr(), _i32(slots).data_ptr(), batch, H, d, dv, _code(qkv), _stream()), "lightning")
+        _i32(seq_lens).data_ptr(), _i32(slots).data_ptr(), batch, H, d, dv, _code(qkv), n_items,
+        _p(None if items is None else _i32(items)), _p(None if first is None else _i32(first)), _p(scratch), _stream()), "lightning")
 
 
 def gated_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:

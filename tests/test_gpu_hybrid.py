@@ -345,6 +345,18 @@ def test_portions_fp32(sizes):
     check(eng_state, FULL, alone("a", toks, sizes), {"a": toks}, FP32_TOL)
 
 
+def test_long_portions_run_as_parallel_chunks_fp32():
+    """Portions long enough for the recurrent layers to cut them into pieces (states joined by a scan): first a long portion
+    from position 0, then a single token, then a long portion that continues from a carried state, beside a short request;
+    lengths off the piece size."""
+    eng_state = engine_for(FULL, torch.float32, max_tokens=1024)
+    a, b = tokens_of(700, FULL["vocab"], 30), tokens_of(6, FULL["vocab"], 31)
+    steps = [[("a", a[:300], False)], [("a", a[300:301], False), ("b", b[:5], False)], [("b", b[5:], True), ("a", a[301:], True)]]
+    got = check(eng_state, FULL, steps, {"a": a, "b": b}, FP32_TOL)
+    whole = replay(eng_state[0], alone("a", a, [257, 443]))["a"]
+    assert rel(got["a"], whole) < 2e-5
+
+
 def test_long_decoding_fp32():
     """A short prompt, then 260 tokens one by one: the recurrent state and the latent rows carry everything."""
     cfg = config([lit(mlp=moe()), lat(mlp=None), lit(heads=2, dim=12, vdim=20)])

@@ -145,7 +145,12 @@ def kernel_rooflines(name: str, prompt: int, batch: int, device) -> dict:
         state = torch.zeros(reqs, H, D, D, dtype=torch.float32, device=device)
         decay = torch.full((H,), 0.97, dtype=torch.float32, device=device)
         o = torch.empty(T, H * D, dtype=torch.float32, device=device)
-        us = _time_us(lambda: mixops.lightning(o, qkv, state, decay, cu, seq, rows, reqs))
+        chunks = None
+        if q_len >= 256:  # what the engine's metadata does for long portions: pieces of 128 tokens in parallel
+            n = -(-q_len // 128)
+            items = i32([[b, c * 128, min((c + 1) * 128, q_len)] for b in range(reqs) for c in range(n)]).view(-1)
+            chunks = (items, i32([b * n for b in range(reqs + 1)]), reqs * n)
+        us = _time_us(lambda: mixops.lightning(o, qkv, state, decay, cu, seq, rows, reqs, chunks=chunks))
         flops = 4.0 * T * H * D * D
         byts = 2 * reqs * H * D * D * 4 + T * 3 * H * D * 2 + T * H * D * 4
         out[f"{phase}.lightning"] = {"us": round(us, 1), "tflops": round(flops / us / 1e6, 2), "tb_s": round(byts / us / 1e6, 3),
