@@ -36,9 +36,12 @@ int msgl_mix_abi_version(void);
 int msgl_mix_embed(float* x32, void* h, const void* table, const int* ids, int tokens, int W, int dtype, void* stream);
 
 /* s = alpha * x_in + sum_p gate[t, p] * y[t, p]   (y: [rows, parts, W] in T or null with parts = 0; gate: fp32 [rows, parts] or
- * null = ones);   out = s / sqrt(mean(s^2) + eps) * (1 + w).  Written to x_out (fp32, may alias x_in) and / or h_out (T). */
+ * null = ones);   out = s / sqrt(mean(s^2) + eps) * (1 + w).  Written to x_out (fp32, may alias x_in) and / or h_out (T).
+ * router != null: the normed row (its copy in T) is routed in the same launch -- fp32 logits over E experts, then the selection
+ * of msgl_mix_route -> ids int32 [rows, top], wts fp32 [rows, top]. */
 int msgl_mix_postnorm(const float* x_in, float* x_out, void* h_out, const void* y, int parts, const float* gate, const void* w,
-                      float alpha, float eps, int rows, int W, int dtype, void* stream);
+                      float alpha, float eps, int rows, int W, int dtype, const void* router, const void* bias, int E, int top, int G,
+                      int keep, int* ids, float* wts, void* stream);
 
 /* One projection row per token = [q: H x (d + r) | latent R | shared rotated key part r] (the last two only with has_kv).
  * Writes the rotated query parts into q_abs[t, h, R : R + r] (fp32, rows of R + r) and, with has_kv, the RMS-normed latent

@@ -144,7 +144,7 @@ MIX_SIGNATURES = {
     "msgl_mix_last_error": (C.c_char_p, []),
     "msgl_mix_abi_version": (_i, []),
     "msgl_mix_embed": (_i, [_p, _p, _p, _p, _i, _i, _i, _p]),
-    "msgl_mix_postnorm": (_i, [_p, _p, _p, _p, _i, _p, _p, _f, _f, _i, _i, _i, _p]),
+    "msgl_mix_postnorm": (_i, [_p, _p, _p, _p, _i, _p, _p, _f, _f, _i, _i, _i, _p, _p, _i, _i, _i, _i, _p, _p, _p]),
     "msgl_mix_latent_prep": (_i, [_p, _l, _p, _p, _p, _p, _p, _p, _f, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
     "msgl_mix_latent_attn_workspace_floats": (_i, [_i, _i, _i, _i]),
     "msgl_mix_latent_attn": (_i, [_p, _p, _p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p, _p]),

@@ -94,31 +94,15 @@ __global__ __launch_bounds__(256) void embed_rows_kernel(float* __restrict__ x32
 
 // ------------------------------------------------------------------------------------------------ post-norm
 // One workgroup per token row.  s = alpha * x + sum_p g[p] * y[p] (fp32, p ascending), out = s * rsqrt(mean(s^2) + eps) * (1 + w).
-template <typename T>
+// ROUTE: the row that was just normed is also the router's input (its copy in T): every wave takes every fourth expert's logit
+// (fp32 dot over the row, wave reduction in a fixed order), then one thread runs the selection -- the feed-forward's choices
+// leave the same launch that closes the mixer's residual sum.  Defined after select_experts.
+template <typename T, bool ROUTE>
 __global__ __launch_bounds__(256) void postnorm_kernel(const float* __restrict__ x_in, float* __restrict__ x_out, T* __restrict__ h_out,
                                                        const T* __restrict__ y, int parts, const float* __restrict__ gate,
-                                                       const T* __restrict__ w, float alpha, float eps, int W) {
-  extern __shared__ float srow[];  // W floats + 4
-  float* red = srow + W;
-  const int t = blockIdx.x;
-  float ss = 0.f;
-  for (int i = threadIdx.x; i < W; i += 256) {
-    float s = alpha * x_in[(size_t)t * W + i];
-    for (int p = 0; p < parts; ++p) {
-      const float yv = ld(y + ((size_t)t * parts + p) * W + i);
-      s = gate ? fmaf(gate[(size_t)t * parts + p], yv, s) : s + yv;
-    }
-    srow[i] = s;
-    ss += s * s;
-  }
-  const float tot = block_sum256(ss, red);
-  const float inv = 1.0f / sqrtf(tot / (float)W + eps);
-  for (int i = threadIdx.x; i < W; i += 256) {
-    const float v = srow[i] * inv * (1.0f + ld(w + i));
-    if (x_out) x_out[(size_t)t * W + i] = v;
-    if (h_out) st(h_out + (size_t)t * W + i, v);
-  }
-}
+                                                       const T* __restrict__ w, float alpha, float eps, int W, const T* __restrict__ router,
+                                                       const T* __restrict__ bias, int E, int top, int G, int keep, int* __restrict__ ids,
+                                                       float* __restrict__ wts);
 
 // ------------------------------------------------------------------------------------------------ latent prep
 // One workgroup per token.  proj row = [ q: H x (d + r) | (has_kv) latent R | shared rotated key part r ].
@@ -437,6 +421,61 @@ __global__ __launch_bounds__(256) void gated_norm_kernel(T* __restrict__ out, co
 // so the matrix cores' fp32 accumulation IS the 32-bit router on the token's 16-bit copy).  s = softmax(z); choice = s + bias;
 // experts outside the `keep` best groups (a group's score = its largest choice) are out; the `top` largest choices win (ties:
 // lowest index); weight = s / (sum of chosen s + 1e-20).  Scores live in LDS columns, one per thread.
+// s[e * st] holds the router logits of one token on entry (st = column stride: one column per thread); c is scratch of the
+// same shape, gs of G entries.  Writes the token's `top` expert ids and weights.
+template <typename T>
+__device__ __forceinline__ void select_experts(float* s, float* c, float* gs, int st, const T* __restrict__ bias, int E, int top, int G,
+                                               int keep, int* __restrict__ ids, float* __restrict__ wts) {
+  float mx = -INFINITY;
+  for (int e = 0; e < E; ++e) mx = fmaxf(mx, s[e * st]);
+  float sum = 0.f;
+  for (int e = 0; e < E; ++e) {
+    const float v = expf(s[e * st] - mx);
+    s[e * st] = v;
+    sum += v;
+  }
+  for (int e = 0; e < E; ++e) {
+    const float v = s[e * st] / sum;
+    s[e * st] = v;
+    c[e * st] = v + (bias ? ld(bias + e) : 0.f);
+  }
+  const int per = E / G;
+  if (keep < G) {
+    // a group's score = its largest choice; it stays if fewer than `keep` groups beat it (ties: the lower index wins)
+    for (int g = 0; g < G; ++g) {
+      float best = -INFINITY;
+      for (int e = g * per; e < (g + 1) * per; ++e) best = fmaxf(best, c[e * st]);
+      gs[g * st] = best;
+    }
+    for (int g = 0; g < G; ++g) {
+      const float mine = gs[g * st];
+      int better = 0;
+      for (int o2 = 0; o2 < G; ++o2) better += (gs[o2 * st] > mine) || (gs[o2 * st] == mine && o2 < g);
+      if (better >= keep)
+        for (int e = g * per; e < (g + 1) * per; ++e) c[e * st] = -INFINITY;
+    }
+  }
+  float tot = 0.f;
+  for (int k = 0; k < top; ++k) {
+    int best = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      const float v = c[e * st];
+      if (v > bv) {
+        best = e;
+        bv = v;
+      }
+    }
+    if (best < 0) best = 0;  // unreachable: the host checks top <= keep * (E / G) and choice scores are finite
+    ids[k] = best;
+    const float sv = s[best * st];
+    wts[k] = sv;
+    tot += sv;
+    c[best * st] = -INFINITY;
+  }
+  for (int k = 0; k < top; ++k) wts[k] /= (tot + 1e-20f);
+}
+
 template <typename T>
 __global__ __launch_bounds__(64) void route_kernel(int* __restrict__ ids, float* __restrict__ wts, const float* __restrict__ z,
                                                    const T* __restrict__ bias, int tokens, int E, int top, int G, int keep, int TPB) {
@@ -446,55 +485,56 @@ __global__ __launch_bounds__(64) void route_kernel(int* __restrict__ ids, float*
   float* s = lds + threadIdx.x;             // s[e * TPB]
   float* c = lds + (size_t)E * TPB + threadIdx.x;
   const float* zr = z + (size_t)t * E;
-  float mx = -INFINITY;
-  for (int e = 0; e < E; ++e) mx = fmaxf(mx, zr[e]);
-  float sum = 0.f;
-  for (int e = 0; e < E; ++e) {
-    const float v = expf(zr[e] - mx);
-    s[e * TPB] = v;
-    sum += v;
+#pragma unroll 8
+  for (int e = 0; e < E; ++e) s[e * TPB] = zr[e];
+  select_experts<T>(s, c, c + (size_t)E * TPB, TPB, bias, E, top, G, keep, ids + (size_t)t * top, wts + (size_t)t * top);
+}
+
+template <typename T, bool ROUTE>
+__global__ __launch_bounds__(256) void postnorm_kernel(const float* __restrict__ x_in, float* __restrict__ x_out, T* __restrict__ h_out,
+                                                       const T* __restrict__ y, int parts, const float* __restrict__ gate,
+                                                       const T* __restrict__ w, float alpha, float eps, int W, const T* __restrict__ router,
+                                                       const T* __restrict__ bias, int E, int top, int G, int keep, int* __restrict__ ids,
+                                                       float* __restrict__ wts) {
+  extern __shared__ float srow[];  // W floats + 4 (+ 2 E + G with ROUTE)
+  float* red = srow + W;
+  const int t = blockIdx.x;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += 256) {
+    float s = alpha * x_in[(size_t)t * W + i];
+    for (int p = 0; p < parts; ++p) {
+      const float yv = ld(y + ((size_t)t * parts + p) * W + i);
+      s = gate ? fmaf(gate[(size_t)t * parts + p], yv, s) : s + yv;
+    }
+    srow[i] = s;
+    ss += s * s;
   }
-  for (int e = 0; e < E; ++e) {
-    const float v = s[e * TPB] / sum;
-    s[e * TPB] = v;
-    c[e * TPB] = v + (bias ? ld(bias + e) : 0.f);
-  }
-  const int per = E / G;
-  if (keep < G) {
-    // a group stays if fewer than `keep` groups beat it (ties: the lower index wins)
-    for (int g = 0; g < G; ++g) {
-      float mine = -INFINITY;
-      for (int e = g * per; e < (g + 1) * per; ++e) mine = fmaxf(mine, s[e * TPB] + (bias ? ld(bias + e) : 0.f));
-      int better = 0;
-      for (int o2 = 0; o2 < G; ++o2) {
-        if (o2 == g) continue;
-        float other = -INFINITY;
-        for (int e = o2 * per; e < (o2 + 1) * per; ++e) other = fmaxf(other, s[e * TPB] + (bias ? ld(bias + e) : 0.f));
-        better += (other > mine) || (other == mine && o2 < g);
-      }
-      if (better >= keep)
-        for (int e = g * per; e < (g + 1) * per; ++e) c[e * TPB] = -INFINITY;
+  const float tot = block_sum256(ss, red);
+  const float inv = 1.0f / sqrtf(tot / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const float v = srow[i] * inv * (1.0f + ld(w + i));
+    if (x_out) x_out[(size_t)t * W + i] = v;
+    if (h_out) st(h_out + (size_t)t * W + i, v);
+    if (ROUTE) {
+      T rounded;
+      st(&rounded, v);
+      srow[i] = ld(&rounded);
     }
   }
-  float tot = 0.f;
-  for (int k = 0; k < top; ++k) {
-    int best = -1;
-    float bv = -INFINITY;
-    for (int e = 0; e < E; ++e) {
-      const float v = c[e * TPB];
-      if (v > bv) {
-        best = e;
-        bv = v;
-      }
-    }
-    if (best < 0) best = 0;  // unreachable: the host checks top <= keep * (E / G) and choice scores are finite
-    ids[(size_t)t * top + k] = best;
-    const float sv = s[best * TPB];
-    wts[(size_t)t * top + k] = sv;
-    tot += sv;
-    c[best * TPB] = -INFINITY;
+  if (!ROUTE) return;
+  float* sc = red + 4;
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int e = wave; e < E; e += 4) {
+    const T* wr = router + (size_t)e * W;
+    float acc = 0.f;
+    for (int i = lane; i < W; i += 64) acc = fmaf(srow[i], ld(wr + i), acc);
+    acc = wave_sum(acc);
+    if (lane == 0) sc[e] = acc;
   }
-  for (int k = 0; k < top; ++k) wts[(size_t)t * top + k] /= (tot + 1e-20f);
+  __syncthreads();
+  if (threadIdx.x == 0)
+    select_experts<T>(sc, sc + E, sc + 2 * E, 1, bias, E, top, G, keep, ids + (size_t)t * top, wts + (size_t)t * top);
 }
 
 // ------------------------------------------------------------------------------------------------ expert bucketing
@@ -842,16 +882,32 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict
   for (int vt = 0; vt < VC; ++vt) o[vt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, lsum = 0.f;
   const int* trow = table + (size_t)req_rows[b] * table_stride;
-  for (int j0 = k_begin; j0 < k_end; j0 += kAKT) {
-    __syncthreads();
-    for (int e = threadIdx.x; e < kAKT * KC * 4; e += 256) {
+  // the next tile's rows are requested before the current tile's products: their latency hides under the MFMAs
+  constexpr int NCH = (kAKT * KC * 4 + 255) / 256;
+  Q4 pre[NCH];
+  auto request = [&](int j0) {
+#pragma unroll
+    for (int u = 0; u < NCH; ++u) {
+      const int e = u * 256 + threadIdx.x;
       const int key = e / (KC * 4), ch = e - key * (KC * 4);
       const int j = j0 + key, k = ch * 8;
-      Q4 v{0u, 0u, 0u, 0u};
-      if (j < k_end && k < dk) v = load8(cache + (size_t)trow[j] * dk + k, dk - k, vec != 0);
-      *reinterpret_cast<Q4*>(&sk[key * KS + k]) = v;
+      pre[u] = Q4{0u, 0u, 0u, 0u};
+      if (e < kAKT * KC * 4 && j < k_end && k < dk) pre[u] = load8(cache + (size_t)trow[j] * dk + k, dk - k, vec != 0);
+    }
+  };
+  constexpr bool kAhead = KC <= 10;  // the widest instances have no registers to spare for a tile in flight
+  if (kAhead && k_begin < k_end) request(k_begin);
+  for (int j0 = k_begin; j0 < k_end; j0 += kAKT) {
+    __syncthreads();
+    if (!kAhead) request(j0);
+#pragma unroll
+    for (int u = 0; u < NCH; ++u) {
+      const int e = u * 256 + threadIdx.x;
+      const int key = e / (KC * 4), ch = e - key * (KC * 4);
+      if (e < kAKT * KC * 4) *reinterpret_cast<Q4*>(&sk[key * KS + ch * 8]) = pre[u];
     }
     __syncthreads();
+    if (kAhead && j0 + kAKT < k_end) request(j0 + kAKT);
     if (!wave_live) continue;
 #pragma unroll
     for (int ks = 0; ks < kAKT / 16; ++ks) {
@@ -992,15 +1048,29 @@ int msgl_mix_embed(float* x32, void* h, const void* table, const int* ids, int t
 }
 
 int msgl_mix_postnorm(const float* x_in, float* x_out, void* h_out, const void* y, int parts, const float* gate, const void* w,
-                      float alpha, float eps, int rows, int W, int dtype, void* stream) {
+                      float alpha, float eps, int rows, int W, int dtype, const void* router, const void* bias, int E, int top, int G,
+                      int keep, int* ids, float* wts, void* stream) {
   MIX_REQUIRE(x_in && w && (x_out || h_out) && rows >= 0 && W >= 1 && dtype_ok(dtype), "postnorm: bad arguments");
   MIX_REQUIRE((parts == 0) == (y == nullptr) && parts >= 0, "postnorm: parts = %d does not match y", parts);
+  const bool route = router != nullptr;
+  if (route) {
+    MIX_REQUIRE(ids && wts, "postnorm: a router needs ids and wts");
+    MIX_REQUIRE(E >= 1 && top >= 1 && top <= E && G >= 1 && E % G == 0 && keep >= 1 && keep <= G && top <= keep * (E / G),
+                "postnorm: bad router sizes E %d top %d groups %d keep %d", E, top, G, keep);
+  }
   if (rows == 0) return MSGL_MIX_OK;
-  const size_t lds = (size_t)(W + 4) * sizeof(float);
+  const size_t lds = (size_t)(W + 4 + (route ? 2 * E + G : 0)) * sizeof(float);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)postnorm_kernel<T>, lds) == 0, "postnorm: row of %d does not fit LDS", W);
-             hipLaunchKernelGGL(postnorm_kernel<T>, dim3(rows), dim3(256), lds, s, x_in, x_out, mp<T>(h_out), cp<T>(y), parts, gate,
-                                cp<T>(w), alpha, eps, W);)
+#define PN_LAUNCH(ROUTE)                                                                                                                \
+  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)postnorm_kernel<T, ROUTE>, lds) == 0, "postnorm: row of %d does not fit LDS", W); \
+             hipLaunchKernelGGL((postnorm_kernel<T, ROUTE>), dim3(rows), dim3(256), lds, s, x_in, x_out, mp<T>(h_out), cp<T>(y), parts,   \
+                                gate, cp<T>(w), alpha, eps, W, cp<T>(router), cp<T>(bias), E, top, G, keep, ids, wts);)
+  if (route) {
+    PN_LAUNCH(true)
+  } else {
+    PN_LAUNCH(false)
+  }
+#undef PN_LAUNCH
   MIX_LAUNCHED("postnorm");
   return MSGL_MIX_OK;
 }
@@ -1136,8 +1206,8 @@ int msgl_mix_route(int* ids, float* wts, const float* z, const void* bias, int t
               "route: bad sizes E %d top %d groups %d keep %d", E, top, G, keep);
   if (tokens == 0) return MSGL_MIX_OK;
   int tpb = 64;
-  while (tpb > 1 && (size_t)2 * E * tpb * sizeof(float) > 64 * 1024) tpb >>= 1;
-  const size_t lds = (size_t)2 * E * tpb * sizeof(float);
+  while (tpb > 1 && (size_t)(2 * E + G) * tpb * sizeof(float) > 64 * 1024) tpb >>= 1;
+  const size_t lds = (size_t)(2 * E + G) * tpb * sizeof(float);
   MIX_REQUIRE(lds <= 64 * 1024, "route: too many experts");
   hipStream_t s = static_cast<hipStream_t>(stream);
   DISPATCH_T(dtype, hipLaunchKernelGGL(route_kernel<T>, dim3((tokens + tpb - 1) / tpb), dim3(64), lds, s, ids, wts, z, cp<T>(bias), tokens, E,

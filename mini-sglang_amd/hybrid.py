@@ -302,10 +302,9 @@ class HybridDecoder:
         gated = mixops.gated_norm(o, proj[:, 2 * H * d + H * dv:], L.out_norm, self.cfg.rms_norm_eps)
         return mixops.linear(gated, L.o)
 
-    def _experts(self, L: _Layer, h: torch.Tensor):
-        """-> (per-choice outputs [T, top, W], weights fp32 [T, top]); the sum over choices is the caller's norm's."""
+    def _experts(self, L: _Layer, h: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+        """-> per-choice outputs [T, top, W] of the experts `ids` chose; the weighted sum over choices is the caller's norm's."""
         m, (T, W) = L.spec.mlp, h.shape
-        ids, wts = mixops.route(h, L.router, L.bias, m.top, m.groups, m.keep)
         seg, perm = mixops.moe_sort(ids, m.experts)
         n = T * m.top
         act = torch.empty((n, m.ff), dtype=self.dtype, device=h.device)
@@ -313,7 +312,7 @@ class HybridDecoder:
                        a_div=m.top, act=mixops.ACT_RELU2)
         y = torch.empty((T, m.top, W), dtype=self.dtype, device=h.device)
         mixops.gemm_nt(y, act, L.down, n, W, m.ff, lda=m.ff, ldb=m.ff, ldc=W, groups=m.experts, b_gs=W * m.ff, seg=seg, c_rows=perm)
-        return y, wts
+        return y
 
     def forward(self, ctx: Any, batch: Any, logits_out: Optional[torch.Tensor] = None, layer_outputs: Optional[list] = None) -> torch.Tensor:
         """-> logits [rows, vocab] in the model dtype: at `batch.logit_rows` (token indices) when set, else at every request's
@@ -323,10 +322,13 @@ class HybridDecoder:
         x, h = mixops.embed(self.embed, batch.input_ids)
         for i, L in enumerate(self.layers):
             y = self._latent(i, L, h, ctx, batch) if L.spec.kind == "latent_attention" else self._lightning(i, L, h, ctx, batch)
-            mixops.postnorm(x, L.norm1, eps, y=y, alpha=alpha, x_out=x, h_out=h)
-            if L.spec.mlp is not None:
-                y, wts = self._experts(L, h)
-                mixops.postnorm(x, L.norm2, eps, y=y, gate=wts, alpha=alpha, x_out=x, h_out=h)
+            m = L.spec.mlp
+            # the norm that closes the mixer's sum also routes its output (router logits, choice, weights: one launch)
+            picks = mixops.postnorm(x, L.norm1, eps, y=y, alpha=alpha, x_out=x, h_out=h,
+                                    route=None if m is None else (L.router, L.bias, m.top, m.groups, m.keep))
+            if m is not None:
+                y = self._experts(L, h, picks[0])
+                mixops.postnorm(x, L.norm2, eps, y=y, gate=picks[1], alpha=alpha, x_out=x, h_out=h)
             elif L.norm2 is not None:
                 mixops.postnorm(x, L.norm2, eps, alpha=alpha, x_out=x, h_out=h)
             if layer_outputs is not None:

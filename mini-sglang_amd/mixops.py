@@ -57,9 +57,10 @@ def embed(table: torch.Tensor, ids: torch.Tensor):
 
 def postnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, *, y: Optional[torch.Tensor] = None,
              gate: Optional[torch.Tensor] = None, alpha: float = 1.0, x_out: Optional[torch.Tensor] = None,
-             h_out: Optional[torch.Tensor] = None) -> None:
+             h_out: Optional[torch.Tensor] = None, route=None):
     """s = alpha x + sum_p gate[:, p] y[:, p];  out = rms_unit(s) * (1 + weight) -> x_out (fp32) and / or h_out (weight's dtype).
-    y: [rows, W] or [rows, parts, W]."""
+    y: [rows, W] or [rows, parts, W].  route = (router [E, W], bias [E] | None, top, groups, keep): the normed rows are routed in
+    the same launch -> returns (expert ids int32 [rows, top], weights fp32 [rows, top]), else None."""
     _dev(x, weight, y, gate, x_out, h_out)
     rows, W = x.shape
     assert x.dtype == torch.float32 and x.is_contiguous() and weight.shape == (W,) and weight.is_contiguous()
@@ -71,10 +72,21 @@ def postnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, *, y: Optional[t
         assert gate.dtype == torch.float32 and gate.is_contiguous() and gate.numel() == rows * parts
     for o, dt in ((x_out, torch.float32), (h_out, weight.dtype)):
         assert o is None or (o.shape == (rows, W) and o.is_contiguous() and o.dtype == dt)
-    if rows == 0:
-        return
-    check_mix(mix_lib().msgl_mix_postnorm(x.data_ptr(), _p(x_out), _p(h_out), _p(y), parts, _p(gate), weight.data_ptr(),
-                                          float(alpha), float(eps), rows, W, _code(weight), _stream()), "postnorm")
+    router = bias = ids = wts = None
+    E = top = groups = keep = 0
+    if route is not None:
+        router, bias, top, groups, keep = route
+        _dev(router, bias)
+        E = router.shape[0]
+        assert router.shape == (E, W) and router.is_contiguous() and router.dtype == weight.dtype
+        assert bias is None or (bias.dtype == weight.dtype and bias.shape == (E,) and bias.is_contiguous())
+        ids = torch.empty((rows, top), dtype=torch.int32, device=x.device)
+        wts = torch.empty((rows, top), dtype=torch.float32, device=x.device)
+    if rows:
+        check_mix(mix_lib().msgl_mix_postnorm(x.data_ptr(), _p(x_out), _p(h_out), _p(y), parts, _p(gate), weight.data_ptr(),
+                                              float(alpha), float(eps), rows, W, _code(weight), _p(router), _p(bias), E, top, groups,
+                                              keep, _p(ids), _p(wts), _stream()), "postnorm")
+    return None if route is None else (ids, wts)
 
 
 def latent_prep(proj: torch.Tensor, q_abs: torch.Tensor, cache: Optional[torch.Tensor], out_loc: Optional[torch.Tensor],

@@ -165,7 +165,8 @@ def kernel_rooflines(name: str, prompt: int, batch: int, device) -> dict:
         n = T * top
         act = torch.empty(n, ff, dtype=bf, device=device)
         y = torch.empty(T, top, W, dtype=bf, device=device)
-        us_r = _time_us(lambda: mixops.route(h, router, bias, top, 4, 2))
+        xr, wr, hr = rnd(T, W, dtype=torch.float32), rnd(W, scale=0.1), torch.empty(T, W, dtype=bf, device=device)
+        us_r = _time_us(lambda: mixops.postnorm(xr, wr, 1e-6, y=h, alpha=2.0, x_out=xr, h_out=hr, route=(router, bias, top, 4, 2)))
         us_s = _time_us(lambda: mixops.moe_sort(ids, E))
         us_u = _time_us(lambda: mixops.gemm_nt(act, h, up, n, ff, W, lda=W, ldb=W, ldc=ff, groups=E, b_gs=ff * W, seg=seg, a_rows=perm,
                                                a_div=top, act=mixops.ACT_RELU2))
@@ -176,8 +177,8 @@ def kernel_rooflines(name: str, prompt: int, batch: int, device) -> dict:
         for key, us in (("experts_up", us_u), ("experts_down", us_d)):
             out[f"{phase}.{key}"] = {"us": round(us, 1), "tflops": round(flops / us / 1e6, 2), "tb_s": round(byts / us / 1e6, 3),
                                      "of_roofline": round(max(flops / us / 1e6 / MFMA_TFLOPS, byts / us / 1e6 / HBM_TBS), 4)}
-        out[f"{phase}.route"] = {"us": round(us_r, 1), "tb_s": round((T * W * 2 + E * W * 2) / us_r / 1e6, 3),
-                                 "of_roofline": round((T * W * 2 + E * W * 2) / us_r / 1e6 / HBM_TBS, 4)}
+        rb = T * W * 12 + E * W * 2  # the post-norm's traffic + the router weights once
+        out[f"{phase}.postnorm_route"] = {"us": round(us_r, 1), "tb_s": round(rb / us_r / 1e6, 3), "of_roofline": round(rb / us_r / 1e6 / HBM_TBS, 4)}
         out[f"{phase}.moe_sort"] = {"us": round(us_s, 1)}
         # --- post-norm (fp32 residual in and out, 16-bit sublayer output in, 16-bit copy out)
         x = rnd(T, W, dtype=torch.float32)
