@@ -476,6 +476,80 @@ __device__ __forceinline__ void select_experts(float* s, float* c, float* gs, in
   for (int k = 0; k < top; ++k) wts[k] /= (tot + 1e-20f);
 }
 
+// The same selection by the 64 lanes of one wave over one token (lane owns experts lane, lane + 64, ...): reductions by
+// lane exchange in a fixed order, so the result does not depend on anything but the logits.  s, c: E entries of LDS each, gs: G + top.
+__device__ __forceinline__ float wave_max_f(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+template <typename T>
+__device__ __forceinline__ void select_experts_wave(float* s, float* c, float* gs, const T* __restrict__ bias, int E, int top, int G,
+                                                    int keep, int* __restrict__ ids, float* __restrict__ wts) {
+  const int lane = threadIdx.x & 63;
+  float mx = -INFINITY;
+  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
+  mx = wave_max_f(mx);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += 64) {
+    const float v = expf(s[e] - mx);
+    s[e] = v;
+    sum += v;
+  }
+  sum = wave_sum(sum);
+  for (int e = lane; e < E; e += 64) {
+    const float v = s[e] / sum;
+    s[e] = v;
+    c[e] = v + (bias ? ld(bias + e) : 0.f);
+  }
+  const int per = E / G;
+  if (keep < G) {
+    for (int g = lane; g < G; g += 64) {
+      float best = -INFINITY;
+      for (int e = g * per; e < (g + 1) * per; ++e) best = fmaxf(best, c[e]);
+      gs[g] = best;
+    }
+    for (int g = lane; g < G; g += 64) {
+      const float mine = gs[g];
+      int better = 0;
+      for (int o2 = 0; o2 < G; ++o2) better += (gs[o2] > mine) || (gs[o2] == mine && o2 < g);
+      if (better >= keep)
+        for (int e = g * per; e < (g + 1) * per; ++e) c[e] = -INFINITY;
+    }
+  }
+  float tot = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float bv = -INFINITY;
+    int best = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = c[e];
+      if (v > bv) {
+        bv = v;
+        best = e;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(best, o, 64);
+      if (ov > bv || (ov == bv && oi < best)) {
+        bv = ov;
+        best = oi;
+      }
+    }
+    if (best == 0x7fffffff) best = 0;  // unreachable: the host checks top <= keep * (E / G) and choice scores are finite
+    const float sv = s[best];
+    tot += sv;
+    if (lane == 0) {
+      ids[k] = best;
+      gs[G + k] = sv;  // the chosen scores wait in LDS (in order within the wave) for the sum
+      c[best] = -INFINITY;
+    }
+  }
+  const float inv = 1.0f / (tot + 1e-20f);
+  for (int k = lane; k < top; k += 64) wts[k] = gs[G + k] * inv;
+}
+
 template <typename T>
 __global__ __launch_bounds__(64) void route_kernel(int* __restrict__ ids, float* __restrict__ wts, const float* __restrict__ z,
                                                    const T* __restrict__ bias, int tokens, int E, int top, int G, int keep, int TPB) {
@@ -496,7 +570,7 @@ __global__ __launch_bounds__(256) void postnorm_kernel(const float* __restrict__
                                                        const T* __restrict__ w, float alpha, float eps, int W, const T* __restrict__ router,
                                                        const T* __restrict__ bias, int E, int top, int G, int keep, int* __restrict__ ids,
                                                        float* __restrict__ wts) {
-  extern __shared__ float srow[];  // W floats + 4 (+ 2 E + G with ROUTE)
+  extern __shared__ float srow[];  // W floats + 4 (+ 2 E + G + top with ROUTE)
   float* red = srow + W;
   const int t = blockIdx.x;
   float ss = 0.f;
@@ -525,16 +599,30 @@ __global__ __launch_bounds__(256) void postnorm_kernel(const float* __restrict__
   float* sc = red + 4;
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int e = wave; e < E; e += 4) {
-    const T* wr = router + (size_t)e * W;
-    float acc = 0.f;
-    for (int i = lane; i < W; i += 64) acc = fmaf(srow[i], ld(wr + i), acc);
-    acc = wave_sum(acc);
-    if (lane == 0) sc[e] = acc;
+  // a wave takes experts wave, wave + 4, ...; up to kRouteAcc of them at once, so that one pass over the row has that many
+  // independent weight loads in flight per lane (element order per expert: lane-strided, then the wave reduction: fixed)
+  constexpr int kRouteAcc = 8;
+  for (int e0 = wave; e0 < E; e0 += 4 * kRouteAcc) {
+    float acc[kRouteAcc];
+#pragma unroll
+    for (int a = 0; a < kRouteAcc; ++a) acc[a] = 0.f;
+    for (int i = lane; i < W; i += 64) {
+      const float hv = srow[i];
+#pragma unroll
+      for (int a = 0; a < kRouteAcc; ++a) {
+        const int e = e0 + 4 * a;
+        if (e < E) acc[a] = fmaf(hv, ld(router + (size_t)e * W + i), acc[a]);
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < kRouteAcc; ++a) {
+      const int e = e0 + 4 * a;
+      const float v = wave_sum(acc[a]);
+      if (e < E && lane == 0) sc[e] = v;
+    }
   }
   __syncthreads();
-  if (threadIdx.x == 0)
-    select_experts<T>(sc, sc + E, sc + 2 * E, 1, bias, E, top, G, keep, ids + (size_t)t * top, wts + (size_t)t * top);
+  if (wave == 0) select_experts_wave<T>(sc, sc + E, sc + 2 * E, bias, E, top, G, keep, ids + (size_t)t * top, wts + (size_t)t * top);
 }
 
 // ------------------------------------------------------------------------------------------------ expert bucketing
@@ -1059,7 +1147,7 @@ int msgl_mix_postnorm(const float* x_in, float* x_out, void* h_out, const void* 
                 "postnorm: bad router sizes E %d top %d groups %d keep %d", E, top, G, keep);
   }
   if (rows == 0) return MSGL_MIX_OK;
-  const size_t lds = (size_t)(W + 4 + (route ? 2 * E + G : 0)) * sizeof(float);
+  const size_t lds = (size_t)(W + 4 + (route ? 2 * E + G + top : 0)) * sizeof(float);
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define PN_LAUNCH(ROUTE)                                                                                                                \
   DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)postnorm_kernel<T, ROUTE>, lds) == 0, "postnorm: row of %d does not fit LDS", W); \

@@ -131,6 +131,8 @@ class _Layer:
 
 
 class HybridDecoder:
+    ROUTE_FUSE_MAX_TOKENS = 128
+
     def __init__(self, cfg: HybridConfig, *, dtype: torch.dtype, device: torch.device, tp_rank: int = 0, tp_size: int = 1,
                  seed: int = 42, init_std: float = 0.02, max_position: Optional[int] = None, **_unused: Any) -> None:
         if tp_size != 1:
@@ -323,9 +325,14 @@ class HybridDecoder:
         for i, L in enumerate(self.layers):
             y = self._latent(i, L, h, ctx, batch) if L.spec.kind == "latent_attention" else self._lightning(i, L, h, ctx, batch)
             m = L.spec.mlp
-            # the norm that closes the mixer's sum also routes its output (router logits, choice, weights: one launch)
+            # Few tokens (decode, short portions): the norm that closes the mixer's sum also routes its output -- router logits,
+            # choice and weights leave the same launch.  Many tokens: every token re-reading the router weights costs more than
+            # the launches it saves, so the logits come from the product kernel (weights reused across a 128-token tile).
+            fuse = m is not None and h.shape[0] <= self.ROUTE_FUSE_MAX_TOKENS
             picks = mixops.postnorm(x, L.norm1, eps, y=y, alpha=alpha, x_out=x, h_out=h,
-                                    route=None if m is None else (L.router, L.bias, m.top, m.groups, m.keep))
+                                    route=(L.router, L.bias, m.top, m.groups, m.keep) if fuse else None)
+            if m is not None and not fuse:
+                picks = mixops.route(h, L.router, L.bias, m.top, m.groups, m.keep)
             if m is not None:
                 y = self._experts(L, h, picks[0])
                 mixops.postnorm(x, L.norm2, eps, y=y, gate=picks[1], alpha=alpha, x_out=x, h_out=h)
