@@ -761,8 +761,8 @@ __global__ __launch_bounds__(256) void gemm_nt_kernel(TC* __restrict__ C, const 
 // ------------------------------------------------------------------------------------------------ grouped GEMM on the matrix cores
 // The same contract as gemm_nt_kernel for 16-bit B (weights): A is rounded to bf16 on its way into LDS (it IS bf16 except for
 // the fp32 latent that meets W_uv), products on v_mfma_f32_16x16x32_bf16 with fp32 accumulation.  128 x 128 tile, 4 waves of
-// 64 x 64 (4 x 4 MFMA tiles each), k in steps of 32; the next step's global loads are issued before the current step's
-// MFMAs.  LDS rows are 40 elements apart (80 B): the 16 lanes of a fragment read land on 16 different bank quads.  A wave
+// 64 x 64 (4 x 4 MFMA tiles each), k in steps of 64 (two MFMA k-blocks); the next step's global loads are issued before the
+// current step's MFMAs.  LDS rows are 72 elements apart (144 B): the 16 lanes of a fragment read land on 16 different bank quads.  A wave
 // whose rows lie past the end of a (short) expert segment skips its MFMAs, so a decode step pays for the weight stream only.
 // An output element's k order is fixed, wherever its row sits in a segment: results do not depend on the batch around it.
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -770,7 +770,7 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 struct __attribute__((aligned(16))) Q4 {
   uint32_t x, y, z, w;
 };
-constexpr int kMT = 128, kMK = 32, kMLd = 40;
+constexpr int kMT = 128, kMK = 64, kMLd = 72;
 
 __device__ __forceinline__ uint32_t bf16_bits(float v) {
   bf16_t t;
@@ -819,11 +819,11 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma_kernel(TC* __restrict__ C, c
   TC* Cg = C + (seg ? 0 : g * c_gs);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
-  const int lr = threadIdx.x >> 2, ks = (threadIdx.x & 3) * 8;
-  int64_t a_off[2], b_off[2];
+  const int lr = threadIdx.x >> 3, ks = (threadIdx.x & 7) * 8;  // loader: rows lr + 32 u, eight k from ks
+  int64_t a_off[4], b_off[4];
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    const int ml = m0 + lr + 64 * u, n = n0 + lr + 64 * u;
+  for (int u = 0; u < 4; ++u) {
+    const int ml = m0 + lr + 32 * u, n = n0 + lr + 32 * u;
     a_off[u] = -1;
     if (ml < rows) {
       const int m = row0 + ml;
@@ -831,11 +831,11 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma_kernel(TC* __restrict__ C, c
     }
     b_off[u] = n < N ? (int64_t)n * ldb : -1;
   }
-  Q4 ra[2], rb[2];
+  Q4 ra[4], rb[4];
   auto gload = [&](int k0) {
     const int k = k0 + ks, n = K - k;
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < 4; ++u) {
       ra[u] = (a_off[u] >= 0 && n > 0) ? load8(Ag + a_off[u] + k, n, a_vec != 0) : Q4{0u, 0u, 0u, 0u};
       rb[u] = (b_off[u] >= 0 && n > 0) ? load8(Bg + b_off[u] + k, n, b_vec != 0) : Q4{0u, 0u, 0u, 0u};
     }
@@ -850,23 +850,26 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma_kernel(TC* __restrict__ C, c
   for (int k0 = 0; k0 < K; k0 += kMK) {
     __syncthreads();
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      *reinterpret_cast<Q4*>(&sa[(lr + 64 * u) * kMLd + ks]) = ra[u];
-      *reinterpret_cast<Q4*>(&sb[(lr + 64 * u) * kMLd + ks]) = rb[u];
+    for (int u = 0; u < 4; ++u) {
+      *reinterpret_cast<Q4*>(&sa[(lr + 32 * u) * kMLd + ks]) = ra[u];
+      *reinterpret_cast<Q4*>(&sb[(lr + 32 * u) * kMLd + ks]) = rb[u];
     }
     __syncthreads();
     if (k0 + kMK < K) gload(k0 + kMK);
     if (live_i > 0) {
-      bf16x8_t fb[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        fb[j] = *reinterpret_cast<const bf16x8_t*>(&sb[(wn + j * 16 + (lane & 15)) * kMLd + (lane >> 4) * 8]);
+      for (int kb = 0; kb < kMK / 32; ++kb) {
+        bf16x8_t fb[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (i < live_i) {
-          const bf16x8_t fa = *reinterpret_cast<const bf16x8_t*>(&sa[(wm + i * 16 + (lane & 15)) * kMLd + (lane >> 4) * 8]);
+        for (int j = 0; j < 4; ++j)
+          fb[j] = *reinterpret_cast<const bf16x8_t*>(&sb[(wn + j * 16 + (lane & 15)) * kMLd + kb * 32 + (lane >> 4) * 8]);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j], fa, acc[i][j], 0, 0, 0);
+        for (int i = 0; i < 4; ++i) {
+          if (i < live_i) {
+            const bf16x8_t fa = *reinterpret_cast<const bf16x8_t*>(&sa[(wm + i * 16 + (lane & 15)) * kMLd + kb * 32 + (lane >> 4) * 8]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[j], fa, acc[i][j], 0, 0, 0);
+          }
         }
       }
     }

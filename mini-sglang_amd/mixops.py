@@ -109,7 +109,8 @@ def latent_prep(proj: torch.Tensor, q_abs: torch.Tensor, cache: Optional[torch.T
 
 
 def latent_attn_splits(batch: int, total_q: int, H: int, max_keys: int) -> int:
-    """Key ranges per request for a step with few query rows: enough workgroups to fill the chip, at least 256 keys each.
+    """Key ranges per request for a step with few query rows: enough workgroups to fill the chip, at least 256 keys each (measured: 64-key ranges double the launch's time -- every
+    range pays the query fragments, a partial row and its share of the merge).
     A function of static sizes only (batch, rows, the LONGEST possible key count), so a captured graph keeps its grid."""
     hb = min(H, 64)
     blocks = (-(-total_q // (64 // hb)) + batch) * -(-H // hb)
