@@ -64,6 +64,19 @@ __device__ __forceinline__ void st(bf16_t* p, float v) {  // round to nearest ev
   p->bits = (uint16_t)(u >> 16);
 }
 
+// eight consecutive elements as fp32 (the caller guarantees 16-byte alignment)
+__device__ __forceinline__ void read8(const float* p, float (&f)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+__device__ __forceinline__ void read8(const bf16_t* p, float (&f)[8]) {
+  const uint4 u = *reinterpret_cast<const uint4*>(p);
+  f[0] = __uint_as_float(u.x << 16); f[1] = __uint_as_float(u.x & 0xffff0000u);
+  f[2] = __uint_as_float(u.y << 16); f[3] = __uint_as_float(u.y & 0xffff0000u);
+  f[4] = __uint_as_float(u.z << 16); f[5] = __uint_as_float(u.z & 0xffff0000u);
+  f[6] = __uint_as_float(u.w << 16); f[7] = __uint_as_float(u.w & 0xffff0000u);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
@@ -602,16 +615,35 @@ __global__ __launch_bounds__(256) void postnorm_kernel(const float* __restrict__
   // a wave takes experts wave, wave + 4, ...; up to kRouteAcc of them at once, so that one pass over the row has that many
   // independent weight loads in flight per lane (element order per expert: lane-strided, then the wave reduction: fixed)
   constexpr int kRouteAcc = 8;
+  const bool wide = (W & 7) == 0 && ((uintptr_t)router & 15u) == 0;
   for (int e0 = wave; e0 < E; e0 += 4 * kRouteAcc) {
     float acc[kRouteAcc];
 #pragma unroll
     for (int a = 0; a < kRouteAcc; ++a) acc[a] = 0.f;
-    for (int i = lane; i < W; i += 64) {
-      const float hv = srow[i];
+    if (wide) {  // eight consecutive weights per lane and load: 16 bytes (bf16) or 32 (fp32)
+      for (int i = lane * 8; i < W; i += 512) {
+        float hv[8];
 #pragma unroll
-      for (int a = 0; a < kRouteAcc; ++a) {
-        const int e = e0 + 4 * a;
-        if (e < E) acc[a] = fmaf(hv, ld(router + (size_t)e * W + i), acc[a]);
+        for (int u = 0; u < 8; ++u) hv[u] = srow[i + u];
+#pragma unroll
+        for (int a = 0; a < kRouteAcc; ++a) {
+          const int e = e0 + 4 * a;
+          if (e < E) {
+            float wv[8];
+            read8(router + (size_t)e * W + i, wv);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc[a] = fmaf(hv[u], wv[u], acc[a]);
+          }
+        }
+      }
+    } else {
+      for (int i = lane; i < W; i += 64) {
+        const float hv = srow[i];
+#pragma unroll
+        for (int a = 0; a < kRouteAcc; ++a) {
+          const int e = e0 + 4 * a;
+          if (e < E) acc[a] = fmaf(hv, ld(router + (size_t)e * W + i), acc[a]);
+        }
       }
     }
 #pragma unroll
