@@ -932,18 +932,19 @@ __global__ __launch_bounds__(256) void gemm_nt_mfma_kernel(TC* __restrict__ C, c
 
 // ------------------------------------------------------------------------------------------------ latent attention on the matrix cores
 // bf16 caches.  A workgroup = 64 query rows ((token, head) pairs of one request: QT tokens x HB heads) in 4 waves of 16 rows,
-// one key range (split z of the keys its last token sees).  Keys come through LDS in tiles of 32 rows, row-major, 16-byte
+// one key range (split z of the keys its last token sees).  Keys come through LDS in tiles of 64 rows, row-major, 16-byte
 // padded (fragment reads of 16 rows hit 16 different bank quads).  Per 16-key subtile and wave:
 //   S^T[16 keys x 16 rows] = K . Q^T     KC x v_mfma_f32_16x16x32_bf16   (Q fragments live in registers, rounded to bf16 once)
 //   a lane then holds ONE query row and FOUR keys: the B-operand layout of the second product, so P stays in its lane;
 //   O^T[16 v x 16 rows] += V^T . P^T     VC x v_mfma_f32_16x16x16_bf16, V^T fragments read TRANSPOSED out of the same row-major
 //   key tile (the latent is both key and value): in a 16-lane group, source lane s points at row 4 g + s / 4, columns
 //   4 (s % 4) .. + 3 and ds_read_b64_tr_b16 hands lane j the four keys of column j.
-// Softmax in fp32 per row: tile max across the four lane groups, running (m, l), O rescaled when a row's max moved.
+// Softmax in fp32 per row, one step per 64-key tile: tile max across the four lane groups, running (m, l), O rescaled when
+// a row's max moved.
 // splits > 1 (decode: few rows, many keys): (m, l, O) partials per split, merged by latent_attn_merge_kernel.
 typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 typedef __attribute__((address_space(3))) s16x4_t lds_s16x4_t;
-constexpr int kAKT = 32;
+constexpr int kAKT = 64;
 
 template <int KC, int VC>
 __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
@@ -953,7 +954,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict
                                                                const int* __restrict__ cu_q, int B, int H, int dk, int dv, float scale,
                                                                int QT, int HB, int splits, int vec) {
   constexpr int KS = KC * 32 + 8;
-  __shared__ __attribute__((aligned(16))) uint16_t sk[kAKT * KS];
+  extern __shared__ __attribute__((aligned(16))) uint16_t sk[];  // [kAKT][KS]
   __shared__ int s_req, s_tok0;
   if (threadIdx.x == 0) {
     int g = blockIdx.x, found = -1, tok0 = 0;
@@ -1018,62 +1019,83 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict
       if (e < kAKT * KC * 4 && j < k_end && k < dk) pre[u] = load8(cache + (size_t)trow[j] * dk + k, dk - k, vec != 0);
     }
   };
-  constexpr bool kAhead = KC <= 10;  // the widest instances have no registers to spare for a tile in flight
+  constexpr bool kAhead = KC <= 6;  // the wider instances have no registers to spare for a tile in flight
   if (kAhead && k_begin < k_end) request(k_begin);
   for (int j0 = k_begin; j0 < k_end; j0 += kAKT) {
     __syncthreads();
-    if (!kAhead) request(j0);
+    if (kAhead) {
 #pragma unroll
-    for (int u = 0; u < NCH; ++u) {
-      const int e = u * 256 + threadIdx.x;
-      const int key = e / (KC * 4), ch = e - key * (KC * 4);
-      if (e < kAKT * KC * 4) *reinterpret_cast<Q4*>(&sk[key * KS + ch * 8]) = pre[u];
+      for (int u = 0; u < NCH; ++u) {
+        const int e = u * 256 + threadIdx.x;
+        const int key = e / (KC * 4), ch = e - key * (KC * 4);
+        if (e < kAKT * KC * 4) *reinterpret_cast<Q4*>(&sk[key * KS + ch * 8]) = pre[u];
+      }
+    } else {
+#pragma unroll 4
+      for (int e = threadIdx.x; e < kAKT * KC * 4; e += 256) {
+        const int key = e / (KC * 4), ch = e - key * (KC * 4);
+        const int j = j0 + key, k = ch * 8;
+        Q4 v{0u, 0u, 0u, 0u};
+        if (j < k_end && k < dk) v = load8(cache + (size_t)trow[j] * dk + k, dk - k, vec != 0);
+        *reinterpret_cast<Q4*>(&sk[key * KS + k]) = v;
+      }
     }
     __syncthreads();
     if (kAhead && j0 + kAKT < k_end) request(j0 + kAKT);
     if (!wave_live) continue;
+    // scores of the whole 64-key tile first (four independent MFMA chains), ONE softmax step for the tile (one exchange
+    // across the lane groups, one rescale of O), then the four value products; rows past k_end are zero rows with weight 0
+    constexpr int NKS = kAKT / 16;
+    float sc[NKS][4], mx = -INFINITY;
 #pragma unroll
-    for (int ks = 0; ks < kAKT / 16; ++ks) {
-      if (j0 + ks * 16 >= k_end) break;
+    for (int ks = 0; ks < NKS; ++ks) {
       f32x4_t sacc{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int kc = 0; kc < KC; ++kc) {
         const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(&sk[(ks * 16 + lr) * KS + kc * 32 + lg * 8]);
         sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kc], sacc, 0, 0, 0);
       }
-      float sc[4], mx = -INFINITY;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         const int j = j0 + ks * 16 + 4 * lg + c;
-        sc[c] = (j <= limit && j < k_end) ? sacc[c] * scale : -INFINITY;
-        mx = fmaxf(mx, sc[c]);
+        sc[ks][c] = (j <= limit && j < k_end) ? sacc[c] * scale : -INFINITY;
+        mx = fmaxf(mx, sc[ks][c]);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m, mx);
-      const bool none = m_new == -INFINITY;  // this row has seen no key yet
-      const float corr = none ? 1.f : __expf(m - m_new);
-      float pe[4], ps = 0.f;
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const bool none = m_new == -INFINITY;  // this row has seen no key yet
+    const float corr = none ? 1.f : __expf(m - m_new);
+    float ps = 0.f;
+    s16x4_t pf[NKS];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      float pe[4];
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        pe[c] = none ? 0.f : __expf(sc[c] - m_new);
+        pe[c] = none ? 0.f : __expf(sc[ks][c] - m_new);
         ps += pe[c];
       }
-      lsum = lsum * corr + ps;
-      m = m_new;
-      if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {
-#pragma unroll
-        for (int vt = 0; vt < VC; ++vt) {
-          o[vt][0] *= corr; o[vt][1] *= corr; o[vt][2] *= corr; o[vt][3] *= corr;
-        }
-      }
       const uint32_t p01 = bf16_bits(pe[0]) | (bf16_bits(pe[1]) << 16), p23 = bf16_bits(pe[2]) | (bf16_bits(pe[3]) << 16);
-      const s16x4_t pf = __builtin_bit_cast(s16x4_t, uint2{p01, p23});
+      pf[ks] = __builtin_bit_cast(s16x4_t, uint2{p01, p23});
+    }
+    lsum = lsum * corr + ps;
+    m = m_new;
+    if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {
+#pragma unroll
+      for (int vt = 0; vt < VC; ++vt) {
+        o[vt][0] *= corr; o[vt][1] *= corr; o[vt][2] *= corr; o[vt][3] *= corr;
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      if (j0 + ks * 16 >= k_end) break;
       const uint16_t* vbase = &sk[(ks * 16 + 4 * lg + (lr >> 2)) * KS + 4 * (lr & 3)];
 #pragma unroll
       for (int vt = 0; vt < VC; ++vt) {
         const s16x4_t vf = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(vbase + vt * 16));
-        o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pf, o[vt], 0, 0, 0);
+        o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pf[ks], o[vt], 0, 0, 0);
       }
     }
   }
@@ -1238,7 +1260,9 @@ int msgl_mix_latent_attn(float* out, const float* q_abs, const void* cache, cons
     const int vec = (((uintptr_t)cache & 15u) == 0 && dk % 8 == 0) ? 1 : 0;
 #define ATTN_CASE(KC, VC)                                                                                                              \
   if (dk <= KC * 32 && dv <= VC * 16) {                                                                                                \
-    hipLaunchKernelGGL((latent_attn_mfma_kernel<KC, VC>), grid, dim3(256), 0, s, out, part_o, part_ml, q_abs, cp<bf16_t>(cache), table, \
+    const size_t lds = (size_t)kAKT * (KC * 32 + 8) * sizeof(uint16_t);                                                                \
+    MIX_REQUIRE(ensure_lds((const void*)latent_attn_mfma_kernel<KC, VC>, lds) == 0, "latent_attn: LDS request refused");               \
+    hipLaunchKernelGGL((latent_attn_mfma_kernel<KC, VC>), grid, dim3(256), lds, s, out, part_o, part_ml, q_abs, cp<bf16_t>(cache), table, \
                        table_stride, req_rows, seq_lens, cu_q, batch, H, dk, dv, scale, QT, HB, splits, vec);                          \
     MIX_LAUNCHED("latent_attn (matrix cores)");                                                                                        \
     if (splits > 1) {                                                                                                                  \
