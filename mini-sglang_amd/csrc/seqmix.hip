@@ -1009,20 +1009,26 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict
   // the next tile's rows are requested before the current tile's products: their latency hides under the MFMAs
   constexpr int NCH = (kAKT * KC * 4 + 255) / 256;
   Q4 pre[NCH];
-  auto request = [&](int j0) {
+  // a tile's pool slots are read from the page table one tile ahead into LDS: the row loads never wait for a table load
+  __shared__ int s_slot[2][kAKT];
+  auto request = [&](int j0, int buf) {
 #pragma unroll
     for (int u = 0; u < NCH; ++u) {
       const int e = u * 256 + threadIdx.x;
       const int key = e / (KC * 4), ch = e - key * (KC * 4);
       const int j = j0 + key, k = ch * 8;
       pre[u] = Q4{0u, 0u, 0u, 0u};
-      if (e < kAKT * KC * 4 && j < k_end && k < dk) pre[u] = load8(cache + (size_t)trow[j] * dk + k, dk - k, vec != 0);
+      if (e < kAKT * KC * 4 && j < k_end && k < dk) pre[u] = load8(cache + (size_t)s_slot[buf][key] * dk + k, dk - k, vec != 0);
     }
   };
   constexpr bool kAhead = KC <= 6;  // the wider instances have no registers to spare for a tile in flight
-  if (kAhead && k_begin < k_end) request(k_begin);
-  for (int j0 = k_begin; j0 < k_end; j0 += kAKT) {
+  if (threadIdx.x < kAKT && k_begin + (int)threadIdx.x < k_end) s_slot[0][threadIdx.x] = trow[k_begin + threadIdx.x];
+  __syncthreads();
+  if (kAhead && k_begin < k_end) request(k_begin, 0);
+  int buf = 0;
+  for (int j0 = k_begin; j0 < k_end; j0 += kAKT, buf ^= 1) {
     __syncthreads();
+    if (threadIdx.x < kAKT && j0 + kAKT + (int)threadIdx.x < k_end) s_slot[buf ^ 1][threadIdx.x] = trow[j0 + kAKT + threadIdx.x];
     if (kAhead) {
 #pragma unroll
       for (int u = 0; u < NCH; ++u) {
@@ -1031,17 +1037,17 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict
         if (e < kAKT * KC * 4) *reinterpret_cast<Q4*>(&sk[key * KS + ch * 8]) = pre[u];
       }
     } else {
-#pragma unroll 4
+#pragma unroll 8
       for (int e = threadIdx.x; e < kAKT * KC * 4; e += 256) {
         const int key = e / (KC * 4), ch = e - key * (KC * 4);
         const int j = j0 + key, k = ch * 8;
         Q4 v{0u, 0u, 0u, 0u};
-        if (j < k_end && k < dk) v = load8(cache + (size_t)trow[j] * dk + k, dk - k, vec != 0);
+        if (j < k_end && k < dk) v = load8(cache + (size_t)s_slot[buf][key] * dk + k, dk - k, vec != 0);
         *reinterpret_cast<Q4*>(&sk[key * KS + k]) = v;
       }
     }
     __syncthreads();
-    if (kAhead && j0 + kAKT < k_end) request(j0 + kAKT);
+    if (kAhead && j0 + kAKT < k_end) request(j0 + kAKT, buf ^ 1);
     if (!wave_live) continue;
     // scores of the whole 64-key tile first (four independent MFMA chains), ONE softmax step for the tile (one exchange
     // across the lane groups, one rescale of O), then the four value products; rows past k_end are zero rows with weight 0
@@ -1131,21 +1137,26 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict
 // out[row] = sum_z e^(m_z - m*) o_z / sum_z e^(m_z - m*) l_z, splits in order; a split without keys has l = 0 and m = -inf
 __global__ __launch_bounds__(64) void latent_attn_merge_kernel(float* __restrict__ out, const float* __restrict__ part_o,
                                                                const float* __restrict__ part_ml, int splits, int dv) {
+  __shared__ float sw[1024];  // per split: its max, then its weight e^(m_z - m*)
+  __shared__ float sl[1024];
   const size_t row = blockIdx.x;
-  float ms = -INFINITY;
-  for (int z = 0; z < splits; ++z) ms = fmaxf(ms, part_ml[(row * splits + z) * 2]);
-  float l = 0.f;
-  for (int z = 0; z < splits; ++z) {
-    const float mz = part_ml[(row * splits + z) * 2];
-    if (mz > -INFINITY) l += part_ml[(row * splits + z) * 2 + 1] * __expf(mz - ms);
+  for (int z = threadIdx.x; z < splits; z += 64) {  // every (m, l) pair is read from memory once
+    sw[z] = part_ml[(row * splits + z) * 2];
+    sl[z] = part_ml[(row * splits + z) * 2 + 1];
   }
+  __syncthreads();
+  float ms = -INFINITY;
+  for (int z = 0; z < splits; ++z) ms = fmaxf(ms, sw[z]);
+  float l = 0.f;
+  for (int z = 0; z < splits; ++z) l += sw[z] > -INFINITY ? sl[z] * __expf(sw[z] - ms) : 0.f;
+  __syncthreads();
+  for (int z = threadIdx.x; z < splits; z += 64) sw[z] = sw[z] > -INFINITY ? __expf(sw[z] - ms) : 0.f;
+  __syncthreads();
   const float inv = 1.0f / l;
   for (int v = threadIdx.x; v < dv; v += 64) {
     float acc = 0.f;
-    for (int z = 0; z < splits; ++z) {
-      const float mz = part_ml[(row * splits + z) * 2];
-      if (mz > -INFINITY) acc += part_o[(row * splits + z) * dv + v] * __expf(mz - ms);
-    }
+#pragma unroll 8
+    for (int z = 0; z < splits; ++z) acc = fmaf(part_o[(row * splits + z) * dv + v], sw[z], acc);
     out[row * dv + v] = acc * inv;
   }
 }
