@@ -6,15 +6,20 @@
 // are stored in the model dtype T (bf16 or fp32).  With T = float every kernel here is true 32-bit.
 //
 //   embed_rows_kernel        x32[t] = table[id[t]]  (+ the T copy the first projection reads)
-//   postnorm_kernel          x32 <- rms(alpha * x32 + sum_p g[t,p] * y[t,p]) * (1 + w)   (+ T copy); also the final norm
+//   postnorm_kernel          x32 <- rms(alpha * x32 + sum_p g[t,p] * y[t,p]) * (1 + w)   (+ T copy); also the final norm;
+//                            ROUTE: router logits, softmax, group-limited top-k and weights of the row it just normed
 //   latent_prep_kernel       latent row: rms-norm(c) | rotate(k_r) -> cache[out_loc];  rotate(q_r) -> q_abs tail
-//   latent_attn_kernel       one shared (c | k_r) key row for all heads, online softmax, output in latent space
-//   lightning_kernel         S <- decay * S + k v^T, o = S^T q per (request, head), state rows indexed by slot
+//   latent_attn_mfma_kernel  bf16 caches: one shared (c | k_r) key row for all heads through LDS, both products on the matrix
+//                            cores, fp32 online softmax, output in latent space; key ranges + latent_attn_merge_kernel for decode
+//   latent_attn_kernel       the same in plain fp32 (fp32 caches, shapes past the matrix-core instances)
+//   lightning_kernel         S <- decay * S + k v^T, o = S^T q per (request, head), state rows indexed by slot; long portions
+//                            as parallel chunks joined by lightning_scan_kernel
 //   gated_norm_kernel        rms over the concatenated heads * w * sigmoid(g)
 //   route_kernel             fp32 router on fp32 logits: softmax, bias-corrected group-limited top-k, normalised weights
 //   moe_count / moe_place    (token, choice) pairs bucketed by expert -> segment offsets + permutation
-//   gemm_nt_kernel           grouped / segmented / gathered C = act(A B^T): per-head latent products, expert layers,
-//                            and every shape the library refuses
+//   gemm_nt_mfma_kernel      grouped / segmented / gathered C = act(A B^T) for 16-bit weights on the matrix cores: per-head
+//                            latent products, expert layers, router logits of long batches
+//   gemm_nt_kernel           the same in fp32 FMA: fp32 engines, and every shape the library refuses
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdint.h>

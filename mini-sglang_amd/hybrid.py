@@ -13,9 +13,10 @@ latent attention   q = W_q h per head [d unrotated | r rotated];  W_dkv h = [lat
                    reads the rows another layer wrote in the same forward.
 lightning          S <- decay_h S + k v^T, o = S^T q with q, k, v = SiLU(projections); fp32 state per (request, head) in the
                    cache's state rows; heads concatenated, RMS-normed (plain weight), gated by sigmoid(W_g h).
-feed-forward       fp32 router (softmax, bias-corrected choice, group-limited top-k), (token, choice) pairs bucketed by expert
-                   on the device, two segmented grouped products (up with ReLU^2, down), the weighted sum of a token's choices
-                   folded into the norm that follows.
+feed-forward       fp32 router (softmax, bias-corrected choice, group-limited top-k) inside the launch of the norm before it
+                   (short batches) or on product-kernel logits (long ones), (token, choice) pairs bucketed by expert on the
+                   device, two segmented grouped products (up with ReLU^2, down), the weighted sum of a token's choices folded
+                   into the norm that follows.
 
 Kernels: csrc/seqmix.hip through mixops.py; plain projections through the library GEMM (mixops.linear).
 """

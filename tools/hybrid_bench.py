@@ -4,7 +4,7 @@ width, depth, head count and ACTIVE feed-forward width, and each sequence-mixing
 
 Random weights, synthetic token ids, bf16.  One JSON line on stdout; does not touch bench.py's default workload.
 
-    python bench.py --hybrid [--hybrid-sizes s m] [--hybrid-prompt 4096] [--hybrid-batch 64] [--hybrid-steps 20]
+    python bench.py --hybrid [--hybrid-args --sizes s m --prompt 2048 --batch 32 --steps 20 --no-dense --no-kernels]
 """
 from __future__ import annotations
 
