@@ -465,3 +465,43 @@ def test_sampled_generation_runs():
     for st in run.last_states:
         out = run.output_ids(st)
         assert len(out) == 6 and all(0 <= t < FULL["vocab"] for t in out)
+
+
+def test_trace_command_line(tmp_path):
+    """bin/trace_run end to end in its own process: a checkpoint folder written here (config.json + safetensors, widths that
+    are no multiple of 16 so that some projections leave the library), recorded steps on stdin, logits files and `done` lines
+    out; fp32 against the restatement, and float32 refused for nothing."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    import numpy as np
+    from safetensors.torch import save_file
+
+    from mini_sglang_amd.hybrid import HybridConfig, HybridDecoder
+
+    cfg = config([lat(heads=3, dim=10, rot_dim=6, vdim=14, kv_rank=22, mlp=moe(experts=6, top=2, ff=26, count=3, keep=2)),
+                  lit(heads=3, dim=10, vdim=18), lat(kv_from=0, heads=2, dim=10, rot_dim=6, vdim=30, kv_rank=22)], width=100, vocab=131)
+    model = HybridDecoder(HybridConfig.from_json(cfg), dtype=torch.bfloat16, device=torch.device("cpu"), seed=9, max_position=64)
+    state = model.export_state()
+    mdir, out = tmp_path / "model", tmp_path / "out"
+    mdir.mkdir()
+    (mdir / "config.json").write_text(json.dumps(cfg))
+    save_file(state, str(mdir / "model.safetensors"))
+    a, b = tokens_of(45, cfg["vocab"], 70), tokens_of(9, cfg["vocab"], 71)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:30], "want": [0, 29]}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": b[:8], "want": []}, {"id": "a", "tokens": a[30:31], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[31:], "want": [13]}, {"id": "b", "tokens": b[8:], "want": [0]}], "end": ["a", "b"]}]
+    root = Path(__file__).resolve().parent.parent
+    pr = subprocess.run([sys.executable, str(root / "bin" / "trace_run"), "--model", str(mdir), "--dtype", "float32", "--out", str(out),
+                         "--max-tokens", "128"], input="\n".join(json.dumps(s) for s in steps) + "\n", text=True, capture_output=True,
+                        timeout=110)
+    assert pr.returncode == 0, pr.stderr[-2000:]
+    assert [ln for ln in pr.stdout.splitlines() if ln.startswith("done")] == ["done 0", "done 1", "done 2"]
+    ra, rb = O.forward(cfg, state, a), O.forward(cfg, state, b)
+    got0 = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4").reshape(2, -1)).double()
+    got1 = torch.from_numpy(np.fromfile(out / "1.f32", dtype="<f4").reshape(1, -1)).double()
+    got2 = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(2, -1)).double()
+    assert rel(got0, ra[[0, 29]]) < FP32_TOL and rel(got1, ra[[30]]) < FP32_TOL
+    assert rel(got2, torch.stack([ra[44], rb[8]])) < FP32_TOL
