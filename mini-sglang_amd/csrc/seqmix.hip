@@ -173,6 +173,37 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const T* __restrict__ 
 }
 
 // ------------------------------------------------------------------------------------------------ latent attention
+// Which request and which of its QT-token groups workgroup `blockIdx.x` owns: group counts ceil(new tokens / QT) of up to 256
+// requests at a time, scanned by the whole workgroup (one pass of independent loads instead of one thread walking the batch).
+// Leaves request -1 for workgroups past the last group.  cnt: 256 ints of LDS; every thread of the (256-thread) workgroup calls.
+__device__ __forceinline__ void find_group(const int* __restrict__ cu_q, int B, int QT, int* cnt, int* s_req, int* s_tok0) {
+  const int tid = threadIdx.x;
+  if (tid == 0) *s_req = -1;
+  int base = 0;
+  for (int c0 = 0; c0 < B; c0 += 256) {
+    const int b = c0 + tid;
+    const int g = b < B ? (cu_q[b + 1] - cu_q[b] + QT - 1) / QT : 0;
+    cnt[tid] = g;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+      const int v = tid >= off ? cnt[tid - off] : 0;
+      __syncthreads();
+      cnt[tid] += v;
+      __syncthreads();
+    }
+    const int incl = cnt[tid], total = cnt[255];
+    const int target = (int)blockIdx.x - base;
+    if (b < B && target >= incl - g && target < incl) {
+      *s_req = b;
+      *s_tok0 = (target - (incl - g)) * QT;
+    }
+    __syncthreads();
+    if (target < total) break;
+    base += total;
+  }
+  __syncthreads();
+}
+
 // Query rows are (token, head) pairs; all heads read the same key row (latent R | rotated r) and the same value row
 // (the latent).  A workgroup = 16 query rows (QT tokens of one request x HB heads) x 16 lanes; keys in tiles of KT through
 // LDS as fp32; online softmax per row in fp32; output = softmax-weighted latent, fp32.
@@ -190,23 +221,8 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(float* __restrict__ ou
   float* sq = lds;                       // [16][dk + 1]
   float* sk = sq + kAttnRows * qs;       // [KT][dk + 1]
   float* sp = sk + KT * qs;              // [16][KT]
-  __shared__ int s_req, s_tok0;
-  if (threadIdx.x == 0) {
-    int g = blockIdx.x, b = 0, found = -1, tok0 = 0;
-    for (; b < B; ++b) {
-      const int n = cu_q[b + 1] - cu_q[b];
-      const int groups = (n + QT - 1) / QT;
-      if (g < groups) {
-        found = b;
-        tok0 = g * QT;
-        break;
-      }
-      g -= groups;
-    }
-    s_req = found;
-    s_tok0 = tok0;
-  }
-  __syncthreads();
+  __shared__ int s_req, s_tok0, s_cnt[256];
+  find_group(cu_q, B, QT, s_cnt, &s_req, &s_tok0);
   const int b = s_req;
   if (b < 0) return;
   const int q_len = cu_q[b + 1] - cu_q[b];
@@ -960,23 +976,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict
                                                                int QT, int HB, int splits, int vec) {
   constexpr int KS = KC * 32 + 8;
   extern __shared__ __attribute__((aligned(16))) uint16_t sk[];  // [kAKT][KS]
-  __shared__ int s_req, s_tok0;
-  if (threadIdx.x == 0) {
-    int g = blockIdx.x, found = -1, tok0 = 0;
-    for (int b = 0; b < B; ++b) {
-      const int n = cu_q[b + 1] - cu_q[b];
-      const int groups = (n + QT - 1) / QT;
-      if (g < groups) {
-        found = b;
-        tok0 = g * QT;
-        break;
-      }
-      g -= groups;
-    }
-    s_req = found;
-    s_tok0 = tok0;
-  }
-  __syncthreads();
+  __shared__ int s_req, s_tok0, s_cnt[256];
+  find_group(cu_q, B, QT, s_cnt, &s_req, &s_tok0);
   const int b = s_req;
   if (b < 0) return;
   const int q_len = cu_q[b + 1] - cu_q[b];
@@ -1042,13 +1043,37 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(float* __restrict
         if (e < kAKT * KC * 4) *reinterpret_cast<Q4*>(&sk[key * KS + ch * 8]) = pre[u];
       }
     } else {
+      // batches of up to 8 row pieces per thread: all loads of a batch are issued before its first LDS store (a store that
+      // waits for its load would hold back the next piece's slot read behind it: LDS operations of a wave stay in order)
+      constexpr int kBatch = 8;
+      if constexpr (KC > 10) {  // the widest instances have no registers for a batch: piece by piece
 #pragma unroll 8
-      for (int e = threadIdx.x; e < kAKT * KC * 4; e += 256) {
-        const int key = e / (KC * 4), ch = e - key * (KC * 4);
-        const int j = j0 + key, k = ch * 8;
-        Q4 v{0u, 0u, 0u, 0u};
-        if (j < k_end && k < dk) v = load8(cache + (size_t)s_slot[buf][key] * dk + k, dk - k, vec != 0);
-        *reinterpret_cast<Q4*>(&sk[key * KS + k]) = v;
+        for (int e = threadIdx.x; e < kAKT * KC * 4; e += 256) {
+          const int key = e / (KC * 4), ch = e - key * (KC * 4);
+          const int j = j0 + key, k = ch * 8;
+          Q4 v{0u, 0u, 0u, 0u};
+          if (j < k_end && k < dk) v = load8(cache + (size_t)s_slot[buf][key] * dk + k, dk - k, vec != 0);
+          *reinterpret_cast<Q4*>(&sk[key * KS + k]) = v;
+        }
+      } else
+#pragma unroll
+      for (int u0 = 0; u0 < NCH; u0 += kBatch) {
+        Q4 tmp[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          const int e = (u0 + u) * 256 + threadIdx.x;
+          const int key = e / (KC * 4), ch = e - key * (KC * 4);
+          const int j = j0 + key, k = ch * 8;
+          tmp[u] = Q4{0u, 0u, 0u, 0u};
+          if (u0 + u < NCH && e < kAKT * KC * 4 && j < k_end && k < dk)
+            tmp[u] = load8(cache + (size_t)s_slot[buf][key] * dk + k, dk - k, vec != 0);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+          const int e = (u0 + u) * 256 + threadIdx.x;
+          const int key = e / (KC * 4), ch = e - key * (KC * 4);
+          if (u0 + u < NCH && e < kAKT * KC * 4) *reinterpret_cast<Q4*>(&sk[key * KS + ch * 8]) = tmp[u];
+        }
       }
     }
     __syncthreads();
