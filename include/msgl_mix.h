@@ -1,6 +1,6 @@
 /*
  * msgl_mix.h -- C ABI of the sequence-mixing kernels (latent attention, linear-recurrence layers, routed experts)
- * for gfx950; implemented by libmsgl_mix.so (mini-sglang_amd/csrc/seqmix.hip).
+ * for gfx950; implemented by libmsgl_mix.so (mini-sglang_amd/csrc/seqmix.hip, mix_delta.hip).
  *
  * Same conventions as msgl_hip.h: raw device pointers, explicit sizes and strides in ELEMENTS, `stream` is a
  * hipStream_t passed as void*, every function returns 0 or a negative code and leaves a message for
@@ -27,7 +27,7 @@ extern "C" {
 #define MSGL_MIX_ACT_NONE 0
 #define MSGL_MIX_ACT_RELU2 1 /* max(z, 0)^2 */
 
-#define MSGL_MIX_ABI_VERSION 1
+#define MSGL_MIX_ABI_VERSION 2
 
 const char* msgl_mix_last_error(void);
 int msgl_mix_abi_version(void);
@@ -94,6 +94,67 @@ int msgl_mix_moe_sort(int* seg, int* perm, int* counts, const int* ids, int n, i
 int msgl_mix_gemm_nt(void* C, const void* A, const void* B, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int groups,
                      int64_t a_gs, int64_t b_gs, int64_t c_gs, const int* seg, const int* a_rows, int a_div, const int* c_rows, int act,
                      int ta, int tb, int tc, void* stream);
+
+/* ---- pre-norm hybrid decoders: windowed attention with mixed heads, gated delta-rule layers, depth-averaged stream ---- */
+
+/* x32[t] = table[ids[t]] / sqrt(mean(row^2) + eps) * w  (fp32). */
+int msgl_mix_embed_norm(float* x32, const void* table, const int* ids, const void* w, float eps, int tokens, int W, int dtype,
+                        void* stream);
+
+/* s = x_in + sum_p gate[t, p] * y[t, p]  (y: [rows, parts, W] in T or null with parts = 0; gate: fp32 or null = ones) -> sum_out
+ * (fp32, may be null).  n_mix > 0: the row that goes on is sum_{j < n_mix - 1} mix_w[j] * hist[j * hist_stride + t * W ..] +
+ * mix_w[n_mix - 1] * s -> x_out (sum_out may be the next row of hist).  w != null: h_out = row / sqrt(mean(row^2) + eps) * w in T.
+ * router != null: the normed row (its copy in T) is routed in the same launch: logits = router row . h + bias, the `top`
+ * largest logits win, wts = softmax over the winners' logits. */
+int msgl_mix_prenorm(const float* x_in, const void* y, int parts, const float* gate, float* sum_out, const float* hist,
+                     int64_t hist_stride, const float* mix_w, int n_mix, float* x_out, const void* w, void* h_out, float eps, int rows,
+                     int W, int dtype, const void* router, const void* bias, int E, int top, int* ids, float* wts, void* stream);
+
+/* out = c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3 over rows of N (powers element-wise, N(.) = the row divided by its root mean
+ * square, eps inside the root); coef: 4 floats on the device. */
+int msgl_mix_poly_act(void* out, const void* z, int64_t ldz, const float* coef, float eps, int rows, int N, int dtype, void* stream);
+
+/* out[r, i] = silu(gate_up[r, i]) * gate_up[r, N + i]  (rows of 2 N -> rows of N). */
+int msgl_mix_silu_mul(void* out, const void* gate_up, int rows, int N, int dtype, void* stream);
+
+/* Router on fp32 logits z [tokens, E] (+ bias in T, may be null): ids = the `top` largest logits (ties: lowest index, in
+ * descending order), wts = softmax over those logits only. */
+int msgl_mix_route_top(int* ids, float* wts, const float* z, const void* bias, int tokens, int E, int top, int dtype, void* stream);
+
+/* Cache rows of a key/value attention layer: k = src[t, k_off : +nk] -> k_cache[out_loc[t]], v = src[t, v_off : +nv] ->
+ * v_cache[out_loc[t]]; with v_first the stored v is (1 - lam) v + lam v_first[t]  (lam: one number in T on the device). */
+int msgl_mix_kv_store(void* k_cache, void* v_cache, const int* out_loc, const void* src, int64_t ld_src, int k_off, int v_off, int nk,
+                      int nv, const void* v_first, int64_t ld_first, const void* lam, int tokens, int dtype, void* stream);
+
+/* Causal attention over the last `window` keys (0 = all) with the heads' scores mixed before the softmax:
+ * s_h(i, j) = scale * sum_g talk[h, g] q_g(i) . k_group(g)(j), softmax over visible j in fp32, o_h = sum_j p_h(j) v_group(h)(j),
+ * out[t, h] = o_h * sigmoid(src[t, g_off + h]) in T.  q = src[t, 0 : H d]; cache rows [slots, G d] / [slots, G dv]; requests as in
+ * msgl_mix_latent_attn (table rows of token slots, seq_lens = keys after this forward, cu_q = prefix of new tokens). */
+int msgl_mix_window_attn(void* out, const void* src, int64_t ld_src, int g_off, const void* k_cache, const void* v_cache, const int* table,
+                         int64_t table_stride, const int* req_rows, const int* seq_lens, const int* cu_q, int batch, int total_q, int H,
+                         int G, int d, int dv, int window, float scale, const float* talk, int dtype, void* stream);
+
+/* Causal convolution over time per channel, then SiLU: out[t, c] = silu(sum_j taps[c, j] in[pos - (n - 1) + j, c]) (fp32);
+ * inputs of this forward are src[t, 0 : C], earlier ones come from state[slots[b]] ([n - 1, C] in T per request: the inputs
+ * of the n - 1 positions before the portion), positions before 0 count as zero.  The first `unit_heads` groups of d channels
+ * leave as unit vectors (x / sqrt(sum x^2 + 1e-6)), the first `scaled_heads` of them times d^-1/2.  A second launch moves every
+ * request's state on to its last n - 1 inputs. */
+int msgl_mix_short_conv(float* out, const void* src, int64_t ld_src, const void* taps, void* state, const int* cu_q, const int* seq_lens,
+                        const int* slots, int batch, int total, int C, int n, int unit_heads, int scaled_heads, int d, int dtype,
+                        void* stream);
+
+/* Gated delta rule per (request, head): S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  qkv: fp32 rows
+ * [q: G x d | k: G x d | v: H x dv] (head h reads q/k group h / (H / G)); state: fp32 [slots, H, d, dv], row slots[b], zero for a
+ * request whose first new token is at position 0; beta = sigmoid(b_raw[t, h]); g = exp(rate[h] * softplus(a_raw[t, i] +
+ * dt_bias[i])) with i = h (per_channel = 0: one decay per head) or h * d + channel (per_channel = 1: one per row of S);
+ * rate = -exp(A_log) in fp32.  out: fp32 [tokens, H * dv]. */
+int msgl_mix_delta_rule(float* out, const float* qkv, float* state, const void* b_raw, int64_t ld_b, const void* a_raw, int64_t ld_a,
+                        int per_channel, const float* rate, const float* dt_bias, const int* cu_q, const int* seq_lens, const int* slots,
+                        int batch, int H, int G, int d, int dv, int dtype, void* stream);
+
+/* out[t, h, e] = o[t, h, e] / sqrt(mean_e(o[t, h]^2) + eps) * w[e] * act(gate[t, h * dv + e]); act: 0 = sigmoid, 1 = SiLU. */
+int msgl_mix_head_gated_norm(void* out, const float* o, const void* gate, int64_t ld_gate, const void* w, float eps, int rows, int H,
+                             int dv, int gate_act, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

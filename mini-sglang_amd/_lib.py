@@ -20,7 +20,7 @@ HIP_SO = LIB_DIR / "libmsgl_hip.so"
 COMM_SO = LIB_DIR / "libmsgl_comm.so"
 GEMM_SO = LIB_DIR / "libmsgl_gemm.so"
 MIX_SO = LIB_DIR / "libmsgl_mix.so"
-MIX_ABI_VERSION = 1
+MIX_ABI_VERSION = 2
 
 BF16, FP16, F32 = 0, 1, 2
 UNIQUE_ID_BYTES = 128
@@ -153,6 +153,16 @@ MIX_SIGNATURES = {
     "msgl_mix_route": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
     "msgl_mix_moe_sort": (_i, [_p, _p, _p, _p, _i, _i, _p]),
     "msgl_mix_gemm_nt": (_i, [_p, _p, _p, _i, _i, _i, _l, _l, _l, _i, _l, _l, _l, _p, _p, _i, _p, _i, _i, _i, _i, _p]),
+    "msgl_mix_embed_norm": (_i, [_p, _p, _p, _p, _f, _i, _i, _i, _p]),
+    "msgl_mix_prenorm": (_i, [_p, _p, _i, _p, _p, _p, _l, _p, _i, _p, _p, _p, _f, _i, _i, _i, _p, _p, _i, _i, _p, _p, _p]),
+    "msgl_mix_poly_act": (_i, [_p, _p, _l, _p, _f, _i, _i, _i, _p]),
+    "msgl_mix_silu_mul": (_i, [_p, _p, _i, _i, _i, _p]),
+    "msgl_mix_route_top": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _p]),
+    "msgl_mix_kv_store": (_i, [_p, _p, _p, _p, _l, _i, _i, _i, _i, _p, _l, _p, _i, _i, _p]),
+    "msgl_mix_window_attn": (_i, [_p, _p, _l, _i, _p, _p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i, _p]),
+    "msgl_mix_short_conv": (_i, [_p, _p, _l, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_delta_rule": (_i, [_p, _p, _p, _p, _l, _p, _l, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_head_gated_norm": (_i, [_p, _p, _p, _l, _p, _f, _i, _i, _i, _i, _i, _p]),
 }
 
 

@@ -1,0 +1,653 @@
+// Kernels of the pre-norm hybrid decoders (windowed attention with mixed heads + gated delta-rule layers + dense or
+// routed feed-forwards, depth-averaged residual stream), gfx950, wave = 64 lanes.  Second translation unit of
+// libmsgl_mix.so; C ABI in include/msgl_mix.h.
+//
+// Precision contract (as in seqmix.hip): the residual stream and its history, every norm, attention scores and weights,
+// decays, step sizes, unit vectors, the recurrent state, router logits and expert weights are fp32 in registers and in
+// memory; tensors that feed a matrix product are stored in the model dtype T (bf16 or fp32).  With T = float every kernel
+// here is true 32-bit.
+//
+//   embed_norm_kernel        X_0[t] = rms(table[id[t]]) * w                                   (fp32)
+//   prenorm_kernel           s = x + sum_p g[t,p] y[t,p];  optional depth average over the stored history;  h = rms(.) * w;
+//                            ROUTE: logits of the normed row, top-`top` by logit, softmax over the chosen ones
+//   poly_act_kernel          a N(z) + b N(z^2) + c N(z^3) + e,  N = divide a row by its root mean square
+//   silu_mul_kernel          silu(gate) * up over rows [gate | up]
+//   route_top_kernel         stand-alone router on given fp32 logits (long batches)
+//   kv_store_kernel          k and the (blended) v of a token -> cache rows at out_loc
+//   window_attn_kernel       sliding-window attention over the paged rows: raw scores of all heads, mixed by the H x H table,
+//                            fp32 online softmax, per-head sigmoid output gate; one workgroup per query token
+//   short_conv_kernel        causal per-channel convolution over time + SiLU, inputs before the portion from the request's
+//                            conv state; q / k heads made unit vectors (q also * d^-1/2);  conv_state_kernel shifts the state
+//   delta_rule_kernel        S <- decay S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q   per (request, head); a thread
+//                            owns one value column of S in registers; scalar or per-key-channel decay
+//   head_gated_norm_kernel   per-head rms over dv * w * (sigmoid | silu)(gate)
+#include "mix_common.h"
+
+namespace {
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float siluf_(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplusf_(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+
+// request of token t: the b with cu_q[b] <= t < cu_q[b + 1]
+__device__ __forceinline__ int request_of(const int* __restrict__ cu_q, int batch, int t) {
+  int lo = 0, hi = batch;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu_q[mid] <= t) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// ------------------------------------------------------------------------------------------------ embedding + norm
+template <typename T>
+__global__ __launch_bounds__(256) void embed_norm_kernel(float* __restrict__ x32, const T* __restrict__ table, const int* __restrict__ ids,
+                                                         const T* __restrict__ w, float eps, int W) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const T* row = table + (size_t)ids[t] * W;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const float v = ld(row + i);
+    ss += v * v;
+  }
+  const float inv = 1.0f / sqrtf(block_sum256(ss, red) / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += 256) x32[(size_t)t * W + i] = ld(row + i) * inv * ld(w + i);
+}
+
+// ------------------------------------------------------------------------------------------------ router on logits
+// s[e * st]: one token's logits (bias already added).  The `top` largest win (ties: lowest index), weights = softmax over them.
+__device__ __forceinline__ void select_top_logits(float* s, int st, int E, int top, int* __restrict__ ids, float* __restrict__ wts) {
+  float first = 0.f, tot = 0.f;
+  for (int k = 0; k < top; ++k) {
+    int best = 0;
+    float bv = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      const float v = s[e * st];
+      if (v > bv) {
+        best = e;
+        bv = v;
+      }
+    }
+    if (k == 0) first = bv;
+    ids[k] = best;
+    const float p = expf(bv - first);
+    wts[k] = p;
+    tot += p;
+    s[best * st] = -INFINITY;
+  }
+  for (int k = 0; k < top; ++k) wts[k] /= tot;
+}
+
+template <typename T>
+__global__ __launch_bounds__(64) void route_top_kernel(int* __restrict__ ids, float* __restrict__ wts, const float* __restrict__ z,
+                                                       const T* __restrict__ bias, int tokens, int E, int top, int TPB) {
+  extern __shared__ float lds[];
+  const int t = blockIdx.x * TPB + threadIdx.x;
+  if (threadIdx.x >= TPB || t >= tokens) return;
+  float* s = lds + threadIdx.x;
+  for (int e = 0; e < E; ++e) s[e * TPB] = z[(size_t)t * E + e] + (bias ? ld(bias + e) : 0.f);
+  select_top_logits(s, TPB, E, top, ids + (size_t)t * top, wts + (size_t)t * top);
+}
+
+// ------------------------------------------------------------------------------------------------ pre-norm, residual sum, depth average
+// One workgroup per token row.  s = x + sum_p g[p] y[p] (fp32, p ascending) -> sum_out;  with n_mix > 0 the row that goes on is
+// sum_{j < n_mix - 1} c[j] hist[j] + c[n_mix - 1] s  (hist: earlier rows of the stream, `hist_stride` floats apart) -> x_out;
+// h = row * rsqrt(mean(row^2) + eps) * w in T.  ROUTE: the normed row (its copy in T) is routed in the same launch.
+template <typename T, bool ROUTE>
+__global__ __launch_bounds__(256) void prenorm_kernel(const float* __restrict__ x_in, const T* __restrict__ y, int parts,
+                                                      const float* __restrict__ gate, float* __restrict__ sum_out,
+                                                      const float* __restrict__ hist, int64_t hist_stride, const float* __restrict__ c,
+                                                      int n_mix, float* __restrict__ x_out, const T* __restrict__ w, T* __restrict__ h_out,
+                                                      float eps, int W, const T* __restrict__ router, const T* __restrict__ bias, int E,
+                                                      int top, int* __restrict__ ids, float* __restrict__ wts) {
+  extern __shared__ float srow[];  // W floats + 4 (+ E with ROUTE)
+  float* red = srow + W;
+  const int t = blockIdx.x;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += 256) {
+    float s = x_in[(size_t)t * W + i];
+    for (int p = 0; p < parts; ++p) {
+      const float yv = ld(y + ((size_t)t * parts + p) * W + i);
+      s = gate ? fmaf(gate[(size_t)t * parts + p], yv, s) : s + yv;
+    }
+    if (sum_out) sum_out[(size_t)t * W + i] = s;
+    if (n_mix > 0) {
+      float m = 0.f;
+      for (int j = 0; j < n_mix - 1; ++j) m = fmaf(c[j], hist[(size_t)j * hist_stride + (size_t)t * W + i], m);
+      s = fmaf(c[n_mix - 1], s, m);
+      if (x_out) x_out[(size_t)t * W + i] = s;
+    }
+    srow[i] = s;
+    ss += s * s;
+  }
+  if (!w) return;
+  const float inv = 1.0f / sqrtf(block_sum256(ss, red) / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += 256) {
+    const float v = srow[i] * inv * ld(w + i);
+    st(h_out + (size_t)t * W + i, v);
+    if (ROUTE) {
+      T rounded;
+      st(&rounded, v);
+      srow[i] = ld(&rounded);
+    }
+  }
+  if (!ROUTE) return;
+  float* sc = red + 4;
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int e = wave; e < E; e += 4) {
+    float acc = 0.f;
+    for (int i = lane; i < W; i += 64) acc = fmaf(srow[i], ld(router + (size_t)e * W + i), acc);
+    acc = wave_sum(acc);
+    if (lane == 0) sc[e] = acc + (bias ? ld(bias + e) : 0.f);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) select_top_logits(sc, 1, E, top, ids + (size_t)t * top, wts + (size_t)t * top);
+}
+
+// ------------------------------------------------------------------------------------------------ activations
+template <typename T>
+__global__ __launch_bounds__(256) void poly_act_kernel(T* __restrict__ out, const T* __restrict__ z, int64_t ldz, const float* __restrict__ coef,
+                                                       float eps, int N) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+  for (int i = threadIdx.x; i < N; i += 256) {
+    const float v = ld(z + (size_t)t * ldz + i), v2 = v * v;
+    s2 += v2;
+    s4 += v2 * v2;
+    s6 += v2 * v2 * v2;
+  }
+  const float n = (float)N;
+  const float i1 = 1.0f / sqrtf(block_sum256(s2, red) / n + eps);
+  const float i2 = 1.0f / sqrtf(block_sum256(s4, red) / n + eps);
+  const float i3 = 1.0f / sqrtf(block_sum256(s6, red) / n + eps);
+  const float a = coef[0] * i1, b = coef[1] * i2, c = coef[2] * i3, e = coef[3];
+  for (int i = threadIdx.x; i < N; i += 256) {
+    const float v = ld(z + (size_t)t * ldz + i);
+    st(out + (size_t)t * N + i, a * v + b * (v * v) + c * (v * v * v) + e);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int64_t total, int N) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int64_t r = i / N;
+  const int col = (int)(i - r * N);
+  const T* row = gu + r * 2 * N;
+  st(out + i, siluf_(ld(row + col)) * ld(row + N + col));
+}
+
+// ------------------------------------------------------------------------------------------------ cache rows of the windowed attention
+// k = src[t, k_off : k_off + nk] -> k_cache[out_loc[t]];  v = src[t, v_off : v_off + nv], blended with the first value-mixing
+// layer's v of the same token when v_first is given: (1 - lam) v + lam v_first  (lam: one number in T on the device).
+template <typename T>
+__global__ __launch_bounds__(256) void kv_store_kernel(T* __restrict__ k_cache, T* __restrict__ v_cache, const int* __restrict__ out_loc,
+                                                       const T* __restrict__ src, int64_t ld_src, int k_off, int v_off, int nk, int nv,
+                                                       const T* __restrict__ v_first, int64_t ld_first, const T* __restrict__ lam) {
+  const int t = blockIdx.x;
+  const size_t slot = (size_t)out_loc[t];
+  const T* row = src + (size_t)t * ld_src;
+  for (int i = threadIdx.x; i < nk; i += 256) k_cache[slot * nk + i] = row[k_off + i];
+  if (v_first) {
+    const float l = ld(lam);
+    for (int i = threadIdx.x; i < nv; i += 256)
+      st(v_cache + slot * nv + i, (1.0f - l) * ld(row + v_off + i) + l * ld(v_first + (size_t)t * ld_first + i));
+  } else {
+    for (int i = threadIdx.x; i < nv; i += 256) v_cache[slot * nv + i] = row[v_off + i];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ windowed attention with mixed heads
+// One workgroup (256 threads) per query token, all H heads.  Keys j with max(0, p - window + 1) <= j <= p in tiles of 64:
+//   raw[g][key] = q_g . k_{group(g)}[key]          thread = (key, every fourth head)
+//   s[h][key]   = scale * sum_g talk[h][g] raw[g][key]
+//   online softmax per head (a wave takes every fourth head, lane = key), p -> LDS
+//   acc[h][e]  = acc * corr[h] + sum_key p[h][key] v_{group(h)}[key][e]       thread = output element (h, e)
+// out[t, h, e] = acc / l[h] * sigmoid(gate[t, h]) in T.
+constexpr int kAttnAcc = 16;  // H * dv <= 256 * kAttnAcc
+
+template <typename T>
+__global__ __launch_bounds__(256) void window_attn_kernel(T* __restrict__ out, const T* __restrict__ src, int64_t ld_src, int g_off,
+                                                          const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                                                          const int* __restrict__ table, int64_t table_stride,
+                                                          const int* __restrict__ req_rows, const int* __restrict__ seq_lens,
+                                                          const int* __restrict__ cu_q, int batch, int H, int G, int d, int dv, int window,
+                                                          float scale, const float* __restrict__ talk) {
+  extern __shared__ float lds[];
+  float* q = lds;                       // H * d
+  float* tk = q + H * d;                // H * H
+  float* raw = tk + H * H;              // H * 64
+  float* pr = raw + H * 64;             // H * 64
+  float* mrow = pr + H * 64;            // H
+  float* lrow = mrow + H;               // H
+  float* corr = lrow + H;               // H
+  int* slots = reinterpret_cast<int*>(corr + H);  // 64
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int b = request_of(cu_q, batch, t);
+  const int n_new = cu_q[b + 1] - cu_q[b];
+  const int p = seq_lens[b] - n_new + (t - cu_q[b]);
+  const int j0 = window > 0 && p - window + 1 > 0 ? p - window + 1 : 0;
+  const int* trow = table + (size_t)req_rows[b] * table_stride;
+  const T* qrow = src + (size_t)t * ld_src;
+  for (int i = tid; i < H * d; i += 256) q[i] = ld(qrow + i);
+  for (int i = tid; i < H * H; i += 256) tk[i] = talk[i] * scale;
+  for (int i = tid; i < H; i += 256) {
+    mrow[i] = -INFINITY;
+    lrow[i] = 0.f;
+  }
+  const int rep = H / G, nk = G * d, nv = G * dv, no = H * dv;
+  float acc[kAttnAcc];
+#pragma unroll
+  for (int a = 0; a < kAttnAcc; ++a) acc[a] = 0.f;
+  const bool wide = (d & 7) == 0;
+  for (int base = j0; base <= p; base += 64) {
+    __syncthreads();
+    if (tid < 64) slots[tid] = base + tid <= p ? trow[base + tid] : -1;
+    __syncthreads();
+    const int slot = slots[lane];
+    for (int g = wave; g < H; g += 4) {
+      float s = 0.f;
+      if (slot >= 0) {
+        const T* kr = k_cache + (size_t)slot * nk + (size_t)(g / rep) * d;
+        const float* qg = q + g * d;
+        if (wide) {
+          for (int i = 0; i < d; i += 8) {
+            float kv[8];
+            read8(kr + i, kv);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s = fmaf(qg[i + u], kv[u], s);
+          }
+        } else {
+          for (int i = 0; i < d; ++i) s = fmaf(qg[i], ld(kr + i), s);
+        }
+      }
+      raw[g * 64 + lane] = s;
+    }
+    __syncthreads();
+    for (int h = wave; h < H; h += 4) {
+      float s = 0.f;
+      for (int g = 0; g < H; ++g) s = fmaf(tk[h * H + g], raw[g * 64 + lane], s);
+      if (slot < 0) s = -INFINITY;
+      const float m_old = mrow[h];
+      const float m_new = fmaxf(m_old, wave_max(s));
+      const float pv = slot < 0 ? 0.f : expf(s - m_new);
+      const float sum = wave_sum(pv);
+      pr[h * 64 + lane] = pv;
+      if (lane == 0) {
+        const float cf = expf(m_old - m_new);
+        corr[h] = cf;
+        lrow[h] = lrow[h] * cf + sum;
+        mrow[h] = m_new;
+      }
+    }
+    __syncthreads();
+    const int keys = p - base + 1 < 64 ? p - base + 1 : 64;
+#pragma unroll
+    for (int a = 0; a < kAttnAcc; ++a) {
+      const int o = tid + 256 * a;
+      if (o < no) {
+        const int h = o / dv, e = o - h * dv;
+        const T* vcol = v_cache + (size_t)(h / rep) * dv + e;
+        const float* ph = pr + h * 64;
+        float s = acc[a] * corr[h];
+        for (int key = 0; key < keys; ++key) s = fmaf(ph[key], ld(vcol + (size_t)slots[key] * nv), s);
+        acc[a] = s;
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int a = 0; a < kAttnAcc; ++a) {
+    const int o = tid + 256 * a;
+    if (o < no) {
+      const int h = o / dv;
+      st(out + (size_t)t * no + o, acc[a] / lrow[h] * sigmoidf_(ld(qrow + g_off + h)));
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ short convolution
+// One workgroup per token.  y[c] = silu(sum_j taps[c][j] in[pos - (n - 1) + j][c]); inputs of this portion come from `src`, earlier
+// ones from the request's conv state (state[slot][s][c] = the input at position start - (n - 1) + s), positions < 0 are zero.
+// The first `unit_heads` groups of d channels are made unit vectors (x / sqrt(sum x^2 + 1e-6)); the first `scaled_heads` of them
+// are also multiplied by d^-1/2.
+template <typename T>
+__global__ __launch_bounds__(256) void short_conv_kernel(float* __restrict__ out, const T* __restrict__ src, int64_t ld_src,
+                                                         const T* __restrict__ taps, const T* __restrict__ state,
+                                                         const int* __restrict__ cu_q, const int* __restrict__ seq_lens,
+                                                         const int* __restrict__ slots, int batch, int C, int n, int unit_heads,
+                                                         int scaled_heads, int d) {
+  extern __shared__ float row[];  // C
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int b = request_of(cu_q, batch, t);
+  const int local = t - cu_q[b];
+  const int pos = seq_lens[b] - (cu_q[b + 1] - cu_q[b]) + local;
+  const T* st_row = state + (size_t)slots[b] * (n - 1) * C;
+  for (int c = tid; c < C; c += 256) {
+    float s = 0.f;
+    for (int j = 0; j < n; ++j) {
+      const int back = n - 1 - j;  // how many tokens before this one
+      if (pos - back < 0) continue;
+      const float x = local - back >= 0 ? ld(src + (size_t)(t - back) * ld_src + c)
+                                        : ld(st_row + (size_t)(n - 1 + local - back) * C + c);
+      s = fmaf(ld(taps + (size_t)c * n + j), x, s);
+    }
+    row[c] = siluf_(s);
+  }
+  __syncthreads();
+  for (int h = wave; h < unit_heads; h += 4) {
+    float ss = 0.f;
+    for (int i = lane; i < d; i += 64) ss = fmaf(row[h * d + i], row[h * d + i], ss);
+    ss = wave_sum(ss);
+    const float f = (h < scaled_heads ? 1.0f / sqrtf((float)d) : 1.0f) / sqrtf(ss + 1e-6f);
+    for (int i = lane; i < d; i += 64) row[h * d + i] *= f;
+  }
+  __syncthreads();
+  for (int c = tid; c < C; c += 256) out[(size_t)t * C + c] = row[c];
+}
+
+// After short_conv_kernel: the state of every request in the batch moves on to its last n - 1 inputs.  Thread = (request, channel).
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_kernel(T* __restrict__ state, const T* __restrict__ src, int64_t ld_src,
+                                                         const int* __restrict__ cu_q, const int* __restrict__ slots, int C, int n) {
+  const int b = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int first = cu_q[b], n_new = cu_q[b + 1] - first;
+  if (n_new <= 0) return;
+  T* sr = state + (size_t)slots[b] * (n - 1) * C + c;
+  constexpr int kMax = 16;
+  T keep[kMax];
+  for (int s = 0; s < n - 1 && s < kMax; ++s) keep[s] = sr[(size_t)s * C];
+  for (int s = 0; s < n - 1; ++s) {
+    const int li = n_new - (n - 1) + s;  // index within the portion of the input that lands in state row s
+    sr[(size_t)s * C] = li >= 0 ? src[(size_t)(first + li) * ld_src + c] : keep[s + n_new];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ gated delta rule
+// Workgroup = (column block of 64, head, request); a thread owns column e of the head's state S [d, dv] (DP >= d registers, the
+// tail zero).  Per token, with g the decay (one number per head, or one per key channel = row of S):
+//   S <- g S;  u = beta (v_e - S^T k);  S <- S + k u;  o_e = S^T q
+// computed as  dk = S_old . (g k), dq = S_old . (g q), u = beta (v_e - dk), S = g S_old + k u, o_e = dq + u (k . q):  the same
+// numbers, one pass less over the column.  q, k (fp32, unit vectors) come from qkv rows [q: G x d | k: G x d | v: H x dv];
+// beta = sigmoid(b_raw[t, h]);  g = exp(rate[h] * softplus(a_raw[t, .] + dt_bias[.])) with rate = -exp(A_log) (fp32, from the host).
+// 16 tokens (8 for the widest heads) are staged in LDS at a time.  A request whose portion starts at position 0 starts from S = 0.
+template <typename T, int DP, bool CHANNEL>
+__global__ __launch_bounds__(64) void delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qkv, float* __restrict__ state,
+                                                        const T* __restrict__ b_raw, int64_t ld_b, const T* __restrict__ a_raw,
+                                                        int64_t ld_a, const float* __restrict__ rate, const float* __restrict__ dt_bias,
+                                                        const int* __restrict__ cu_q, const int* __restrict__ seq_lens,
+                                                        const int* __restrict__ slots, int H, int G, int d, int dv) {
+  constexpr int kStage = DP > 128 ? 8 : 16;
+  __shared__ __attribute__((aligned(16))) float sk[kStage][DP], sgk[kStage][DP], sgq[kStage][DP], sg[kStage][DP];
+  __shared__ float skq[kStage], sbeta[kStage];
+  const int b = blockIdx.z, h = blockIdx.y, e = blockIdx.x * 64 + threadIdx.x, lane = threadIdx.x;
+  const int first = cu_q[b], n_new = cu_q[b + 1] - first;
+  if (n_new <= 0) return;
+  const bool fresh = seq_lens[b] == n_new;
+  const int C = 2 * G * d + H * dv, kvh = h / (H / G);
+  float* Srow = state + ((size_t)slots[b] * H + h) * d * dv;
+  const bool live = e < dv;
+  float S[DP];
+#pragma unroll
+  for (int i = 0; i < DP; ++i) S[i] = (!fresh && live && i < d) ? Srow[(size_t)i * dv + e] : 0.f;
+  const float r = rate[h];
+  for (int t0 = 0; t0 < n_new; t0 += kStage) {
+    const int nt = n_new - t0 < kStage ? n_new - t0 : kStage;
+    __syncthreads();
+    for (int idx = lane; idx < nt * DP; idx += 64) {
+      const int tt = idx / DP, i = idx - tt * DP;
+      const size_t t = (size_t)(first + t0 + tt);
+      float kv = 0.f, qv = 0.f, g = 1.f;
+      if (i < d) {
+        qv = qkv[t * C + kvh * d + i];
+        kv = qkv[t * C + (G + kvh) * d + i];
+        const int ai = CHANNEL ? h * d + i : h;
+        g = expf(r * softplusf_(ld(a_raw + t * ld_a + ai) + dt_bias[ai]));
+      }
+      sk[tt][i] = kv;
+      sgk[tt][i] = g * kv;
+      sgq[tt][i] = g * qv;
+      sg[tt][i] = g;
+    }
+    if (lane < nt) {
+      const size_t t = (size_t)(first + t0 + lane);
+      float kq = 0.f;
+      for (int i = 0; i < d; ++i) kq = fmaf(qkv[t * C + kvh * d + i], qkv[t * C + (G + kvh) * d + i], kq);
+      skq[lane] = kq;
+      sbeta[lane] = sigmoidf_(ld(b_raw + t * ld_b + h));
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const size_t t = (size_t)(first + t0 + tt);
+      const float v = live ? qkv[t * C + 2 * G * d + h * dv + e] : 0.f;
+      float dk = 0.f, dq = 0.f;
+#pragma unroll
+      for (int i = 0; i < DP; ++i) {
+        dk = fmaf(S[i], sgk[tt][i], dk);
+        dq = fmaf(S[i], sgq[tt][i], dq);
+      }
+      const float u = sbeta[tt] * (v - dk);
+#pragma unroll
+      for (int i = 0; i < DP; ++i) S[i] = fmaf(sk[tt][i], u, sg[tt][i] * S[i]);
+      if (live) out[t * (size_t)(H * dv) + h * dv + e] = fmaf(u, skq[tt], dq);
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < DP; ++i)
+      if (i < d) Srow[(size_t)i * dv + e] = S[i];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ per-head gated norm
+// out[t, h, e] = o / sqrt(mean_e(o[t, h]^2) + eps) * w[e] * act(gate[t, h, e]);  act = sigmoid (0) or SiLU (1).  A wave per head.
+template <typename T>
+__global__ __launch_bounds__(256) void head_gated_norm_kernel(T* __restrict__ out, const float* __restrict__ o, const T* __restrict__ g,
+                                                              int64_t ld_g, const T* __restrict__ w, float eps, int H, int dv, int act) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int h = wave; h < H; h += 4) {
+    const float* oh = o + ((size_t)t * H + h) * dv;
+    float ss = 0.f;
+    for (int i = lane; i < dv; i += 64) ss = fmaf(oh[i], oh[i], ss);
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)dv + eps);
+    for (int i = lane; i < dv; i += 64) {
+      const float z = ld(g + (size_t)t * ld_g + h * dv + i);
+      st(out + ((size_t)t * H + h) * dv + i, oh[i] * inv * ld(w + i) * (act ? siluf_(z) : sigmoidf_(z)));
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int msgl_mix_embed_norm(float* x32, const void* table, const int* ids, const void* w, float eps, int tokens, int W, int dtype,
+                        void* stream) {
+  MIX_REQUIRE(x32 && table && ids && w && tokens >= 0 && W >= 1 && dtype_ok(dtype), "embed_norm: bad arguments");
+  if (tokens == 0) return MSGL_MIX_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, hipLaunchKernelGGL(embed_norm_kernel<T>, dim3(tokens), dim3(256), 0, s, x32, cp<T>(table), ids, cp<T>(w), eps, W);)
+  MIX_LAUNCHED("embed_norm");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_prenorm(const float* x_in, const void* y, int parts, const float* gate, float* sum_out, const float* hist,
+                     int64_t hist_stride, const float* mix_w, int n_mix, float* x_out, const void* w, void* h_out, float eps, int rows,
+                     int W, int dtype, const void* router, const void* bias, int E, int top, int* ids, float* wts, void* stream) {
+  MIX_REQUIRE(x_in && rows >= 0 && W >= 1 && dtype_ok(dtype), "prenorm: bad arguments");
+  MIX_REQUIRE((parts == 0) == (y == nullptr) && parts >= 0, "prenorm: parts = %d does not match y", parts);
+  MIX_REQUIRE((w == nullptr) == (h_out == nullptr), "prenorm: a norm weight needs h_out and the reverse");
+  MIX_REQUIRE(n_mix >= 0 && (n_mix == 0 || (mix_w && x_out && (n_mix == 1 || hist))), "prenorm: depth average without its rows");
+  const bool route = router != nullptr;
+  if (route) MIX_REQUIRE(w && ids && wts && E >= 1 && top >= 1 && top <= E, "prenorm: bad router arguments (E %d top %d)", E, top);
+  if (rows == 0) return MSGL_MIX_OK;
+  const size_t lds = (size_t)(W + 4 + (route ? E : 0)) * sizeof(float);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define PRE_LAUNCH(ROUTE)                                                                                                               \
+  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)prenorm_kernel<T, ROUTE>, lds) == 0, "prenorm: row of %d does not fit LDS", W); \
+             hipLaunchKernelGGL((prenorm_kernel<T, ROUTE>), dim3(rows), dim3(256), lds, s, x_in, cp<T>(y), parts, gate, sum_out, hist,  \
+                                hist_stride, mix_w, n_mix, x_out, cp<T>(w), mp<T>(h_out), eps, W, cp<T>(router), cp<T>(bias), E, top,   \
+                                ids, wts);)
+  if (route) {
+    PRE_LAUNCH(true)
+  } else {
+    PRE_LAUNCH(false)
+  }
+#undef PRE_LAUNCH
+  MIX_LAUNCHED("prenorm");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_poly_act(void* out, const void* z, int64_t ldz, const float* coef, float eps, int rows, int N, int dtype, void* stream) {
+  MIX_REQUIRE(out && z && coef && rows >= 0 && N >= 1 && ldz >= N && dtype_ok(dtype), "poly_act: bad arguments");
+  if (rows == 0) return MSGL_MIX_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, hipLaunchKernelGGL(poly_act_kernel<T>, dim3(rows), dim3(256), 0, s, mp<T>(out), cp<T>(z), ldz, coef, eps, N);)
+  MIX_LAUNCHED("poly_act");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_silu_mul(void* out, const void* gate_up, int rows, int N, int dtype, void* stream) {
+  MIX_REQUIRE(out && gate_up && rows >= 0 && N >= 1 && dtype_ok(dtype), "silu_mul: bad arguments");
+  if (rows == 0) return MSGL_MIX_OK;
+  const int64_t total = (int64_t)rows * N;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, hipLaunchKernelGGL(silu_mul_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, mp<T>(out),
+                                       cp<T>(gate_up), total, N);)
+  MIX_LAUNCHED("silu_mul");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_route_top(int* ids, float* wts, const float* z, const void* bias, int tokens, int E, int top, int dtype, void* stream) {
+  MIX_REQUIRE(ids && wts && z && dtype_ok(dtype) && E >= 1 && top >= 1 && top <= E, "route_top: bad arguments (E %d top %d)", E, top);
+  if (tokens == 0) return MSGL_MIX_OK;
+  int tpb = 64;
+  while (tpb > 1 && (size_t)E * tpb * sizeof(float) > 64 * 1024) tpb >>= 1;
+  const size_t lds = (size_t)E * tpb * sizeof(float);
+  MIX_REQUIRE(lds <= 64 * 1024, "route_top: too many experts");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, hipLaunchKernelGGL(route_top_kernel<T>, dim3((tokens + tpb - 1) / tpb), dim3(64), lds, s, ids, wts, z, cp<T>(bias),
+                                       tokens, E, top, tpb);)
+  MIX_LAUNCHED("route_top");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_kv_store(void* k_cache, void* v_cache, const int* out_loc, const void* src, int64_t ld_src, int k_off, int v_off, int nk,
+                      int nv, const void* v_first, int64_t ld_first, const void* lam, int tokens, int dtype, void* stream) {
+  MIX_REQUIRE(k_cache && v_cache && out_loc && src && tokens >= 0 && nk >= 1 && nv >= 1 && k_off >= 0 && v_off >= 0 && dtype_ok(dtype),
+              "kv_store: bad arguments");
+  MIX_REQUIRE(ld_src >= k_off + nk && ld_src >= v_off + nv, "kv_store: columns past the source row");
+  MIX_REQUIRE(!v_first || (lam && ld_first >= nv), "kv_store: value blending needs its factor and rows of at least nv");
+  if (tokens == 0) return MSGL_MIX_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, hipLaunchKernelGGL(kv_store_kernel<T>, dim3(tokens), dim3(256), 0, s, mp<T>(k_cache), mp<T>(v_cache), out_loc,
+                                       cp<T>(src), ld_src, k_off, v_off, nk, nv, cp<T>(v_first), ld_first, cp<T>(lam));)
+  MIX_LAUNCHED("kv_store");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_window_attn(void* out, const void* src, int64_t ld_src, int g_off, const void* k_cache, const void* v_cache, const int* table,
+                         int64_t table_stride, const int* req_rows, const int* seq_lens, const int* cu_q, int batch, int total_q, int H,
+                         int G, int d, int dv, int window, float scale, const float* talk, int dtype, void* stream) {
+  MIX_REQUIRE(out && src && k_cache && v_cache && table && req_rows && seq_lens && cu_q && talk && dtype_ok(dtype),
+              "window_attn: null pointer / dtype");
+  MIX_REQUIRE(batch >= 0 && total_q >= 0 && H >= 1 && G >= 1 && H % G == 0 && d >= 1 && dv >= 1 && window >= 0,
+              "window_attn: bad sizes H %d G %d d %d dv %d window %d", H, G, d, dv, window);
+  MIX_REQUIRE(H * dv <= 256 * kAttnAcc, "window_attn: %d output elements per token (at most %d)", H * dv, 256 * kAttnAcc);
+  MIX_REQUIRE(ld_src >= (int64_t)H * d && ld_src >= g_off + H && g_off >= 0, "window_attn: columns past the source row");
+  MIX_REQUIRE(dtype == MSGL_MIX_F32 || (d % 8 != 0) || ((G * d) % 8 == 0), "window_attn: key rows not 16-byte aligned");
+  if (total_q == 0 || batch == 0) return MSGL_MIX_OK;
+  const size_t lds = (size_t)(H * d + H * H + 2 * H * 64 + 3 * H + 64) * sizeof(float);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)window_attn_kernel<T>, lds) == 0, "window_attn: %zu bytes of LDS", lds);
+             hipLaunchKernelGGL(window_attn_kernel<T>, dim3(total_q), dim3(256), lds, s, mp<T>(out), cp<T>(src), ld_src, g_off,
+                                cp<T>(k_cache), cp<T>(v_cache), table, table_stride, req_rows, seq_lens, cu_q, batch, H, G, d, dv, window,
+                                scale, talk);)
+  MIX_LAUNCHED("window_attn");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_short_conv(float* out, const void* src, int64_t ld_src, const void* taps, void* state, const int* cu_q, const int* seq_lens,
+                        const int* slots, int batch, int total, int C, int n, int unit_heads, int scaled_heads, int d, int dtype,
+                        void* stream) {
+  MIX_REQUIRE(out && src && taps && cu_q && seq_lens && slots && dtype_ok(dtype), "short_conv: null pointer / dtype");
+  MIX_REQUIRE(batch >= 0 && total >= 0 && C >= 1 && n >= 1 && n <= 17 && ld_src >= C && (n == 1 || state),
+              "short_conv: bad sizes C %d taps %d", C, n);
+  MIX_REQUIRE(unit_heads >= 0 && scaled_heads >= 0 && scaled_heads <= unit_heads && d >= 1 && (int64_t)unit_heads * d <= C,
+              "short_conv: unit-vector heads past the row");
+  if (total == 0 || batch == 0) return MSGL_MIX_OK;
+  const size_t lds = (size_t)C * sizeof(float);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)short_conv_kernel<T>, lds) == 0, "short_conv: row of %d does not fit LDS", C);
+             hipLaunchKernelGGL(short_conv_kernel<T>, dim3(total), dim3(256), lds, s, out, cp<T>(src), ld_src, cp<T>(taps), cp<T>(state),
+                                cu_q, seq_lens, slots, batch, C, n, unit_heads, scaled_heads, d);
+             if (n > 1) hipLaunchKernelGGL(conv_state_kernel<T>, dim3((C + 255) / 256, batch), dim3(256), 0, s, mp<T>(state), cp<T>(src),
+                                           ld_src, cu_q, slots, C, n);)
+  MIX_LAUNCHED("short_conv");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_delta_rule(float* out, const float* qkv, float* state, const void* b_raw, int64_t ld_b, const void* a_raw, int64_t ld_a,
+                        int per_channel, const float* rate, const float* dt_bias, const int* cu_q, const int* seq_lens, const int* slots,
+                        int batch, int H, int G, int d, int dv, int dtype, void* stream) {
+  MIX_REQUIRE(out && qkv && state && b_raw && a_raw && rate && dt_bias && cu_q && seq_lens && slots && dtype_ok(dtype),
+              "delta_rule: null pointer / dtype");
+  MIX_REQUIRE(batch >= 0 && H >= 1 && G >= 1 && H % G == 0 && d >= 1 && d <= 256 && dv >= 1, "delta_rule: bad sizes H %d G %d d %d dv %d", H,
+              G, d, dv);
+  MIX_REQUIRE(ld_b >= H && ld_a >= (per_channel ? H * d : H), "delta_rule: rows shorter than their heads");
+  if (batch == 0) return MSGL_MIX_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((dv + 63) / 64, H, batch);
+#define DR_LAUNCH(DP, CH)                                                                                                             \
+  DISPATCH_T(dtype, hipLaunchKernelGGL((delta_rule_kernel<T, DP, CH>), grid, dim3(64), 0, s, out, qkv, state, cp<T>(b_raw), ld_b,     \
+                                       cp<T>(a_raw), ld_a, rate, dt_bias, cu_q, seq_lens, slots, H, G, d, dv);)
+#define DR_CASE(DP)            \
+  if (per_channel) {           \
+    DR_LAUNCH(DP, true)        \
+  } else {                     \
+    DR_LAUNCH(DP, false)       \
+  }
+  if (d <= 16) {
+    DR_CASE(16)
+  } else if (d <= 32) {
+    DR_CASE(32)
+  } else if (d <= 64) {
+    DR_CASE(64)
+  } else if (d <= 96) {
+    DR_CASE(96)
+  } else if (d <= 128) {
+    DR_CASE(128)
+  } else if (d <= 192) {
+    DR_CASE(192)
+  } else {
+    DR_CASE(256)
+  }
+#undef DR_CASE
+#undef DR_LAUNCH
+  MIX_LAUNCHED("delta_rule");
+  return MSGL_MIX_OK;
+}
+
+int msgl_mix_head_gated_norm(void* out, const float* o, const void* gate, int64_t ld_gate, const void* w, float eps, int rows, int H,
+                             int dv, int gate_act, int dtype, void* stream) {
+  MIX_REQUIRE(out && o && gate && w && rows >= 0 && H >= 1 && dv >= 1 && ld_gate >= (int64_t)H * dv && dtype_ok(dtype) &&
+                  (gate_act == 0 || gate_act == 1),
+              "head_gated_norm: bad arguments");
+  if (rows == 0) return MSGL_MIX_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  DISPATCH_T(dtype, hipLaunchKernelGGL(head_gated_norm_kernel<T>, dim3(rows), dim3(256), 0, s, mp<T>(out), o, cp<T>(gate), ld_gate,
+                                       cp<T>(w), eps, H, dv, gate_act);)
+  MIX_LAUNCHED("head_gated_norm");
+  return MSGL_MIX_OK;
+}
+
+}  // extern "C"

@@ -18,7 +18,23 @@ feed-forward       fp32 router (softmax, bias-corrected choice, group-limited to
                    device, two segmented grouped products (up with ReLU^2, down), the weighted sum of a token's choices folded
                    into the norm that follows.
 
-Kernels: csrc/seqmix.hip through mixops.py; plain projections through the library GEMM (mixops.linear).
+A second residual scheme, `pre_norm_depth` (the Bedarax design), runs the same loop with other pieces:
+
+stream             X_0 = rms_unit(embed[token]) * w_e;  per layer  s = x + mixer(norm1(x)),  X_(i+1) = s + ff(norm2(s)),
+                   x <- sum_{j <= i+1} c_i[j] X_j  (every layer averages the whole history with its own weights); norms have
+                   plain weights; the LM head is its own matrix.  The history is one fp32 tensor [layers + 1, tokens, W].
+attention          q, k, v projections without rotation; the heads' scores are mixed by an H x H table before the softmax;
+                   only the last `window` keys are visible; from the second value-mixing layer on, the cached v is blended
+                   with the first such layer's v of the same token; a sigmoid gate per head scales the output.  Cached per
+                   token: k [G d] and the blended v [G dv] in the pool's token slots.
+delta / channel_delta   q, k, v pass a short causal convolution over time (+ SiLU), q and k become unit vectors per head;
+                   S <- g S, u = beta (v - S^T k), S <- S + k u^T, o = S^T q with one decay g per head (delta) or per key
+                   channel through a low-rank projection (channel_delta); per-head RMS norm, gated by SiLU / sigmoid.
+                   State per request: S in fp32 and the last taps - 1 inputs of the convolution.
+feed-forward       dense with a polynomial activation of row-normalised powers, or routed experts silu(W_g h) * (W_u h)
+                   chosen by the largest router logits (softmax over the chosen logits only).
+
+Kernels: csrc/seqmix.hip and csrc/mix_delta.hip through mixops.py; plain projections through the library GEMM (mixops.linear).
 """
 from __future__ import annotations
 
@@ -39,11 +55,20 @@ class MoeSpec:
     ff: int
     groups: int = 1
     keep: int = 1
+    gated: bool = False             # expert = W_down (silu(W_gate h) * (W_up h)) instead of W_down relu(W_up h)^2
+    pick: str = "scores"            # "scores": softmax over all experts, corrected group-limited choice; "logits": the largest
+                                    # logits (+ bias) win and the weights are the softmax over the winners
+
+
+@dataclass(frozen=True)
+class DenseFfSpec:
+    ff: int
+    act: str = "poly_norm"          # c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3 with N = divide a row by its root mean square
 
 
 @dataclass(frozen=True)
 class LayerSpec:
-    kind: str                       # "latent_attention" | "lightning"
+    kind: str                       # "latent_attention" | "lightning" | "attention" | "delta" | "channel_delta"
     heads: int
     dim: int                        # unrotated query/key size per head (lightning: query/key size)
     vdim: int
@@ -55,7 +80,17 @@ class LayerSpec:
     rot_base: float = 10000.0
     rot_scaling: Optional[Tuple[Tuple[str, float], ...]] = None
     decay: Tuple[float, ...] = ()
-    mlp: Optional[MoeSpec] = None
+    mlp: Optional[Any] = None       # MoeSpec | DenseFfSpec | None
+    kv_heads: int = 0               # attention / delta kinds: key (and attention: value) heads; query head h reads h // (heads / kv_heads)
+    window: int = 0                 # attention: keys i - window < j <= i are visible; 0 = all earlier keys
+    v_mix: bool = False             # attention: blends its values with those of the first such layer
+    conv: int = 1                   # delta kinds: taps of the causal convolution over q, k, v
+    decay_rank: int = 0             # channel_delta: inner sizes of the two-step decay and gate projections
+    gate_rank: int = 0
+
+    @property
+    def recurrent(self) -> bool:
+        return self.kind in ("lightning", "delta", "channel_delta")
 
 
 @dataclass(frozen=True)
@@ -65,9 +100,11 @@ class HybridConfig:
     hidden_size: int
     layers: Tuple[LayerSpec, ...]
     rms_norm_eps: float
-    postln_alpha: float
+    postln_alpha: float = 1.0
     max_position: int = 1 << 20
     name: str = "Nidorax"
+    residual: str = "post_norm"     # "post_norm": x <- norm(alpha x + f(x)), weights stored as offsets from one, tied head;
+                                    # "pre_norm_depth": x + f(norm(x)), depth-averaged history, normed embedding, own head
 
     @property
     def num_layers(self) -> int:
@@ -111,6 +148,50 @@ class HybridConfig:
                             rms_norm_eps=float(cfg["norm"]["eps"]), postln_alpha=float(cfg["postln_alpha"]), name=name)
 
 
+def _ff_spec(i: int, mlp: Optional[Dict[str, Any]]):
+    if mlp is None:
+        return None
+    kind = mlp.get("kind")
+    if kind == "dense":
+        return DenseFfSpec(ff=int(mlp["ff"]))
+    if kind == "moe":
+        r = mlp["router"]
+        return MoeSpec(experts=int(r["experts"]), top=int(r["top"]), ff=int(mlp["expert"]["ff"]), gated=True, pick="logits")
+    raise ValueError(f"layer {i}: unknown feed-forward kind {kind!r}")
+
+
+def bedarax_config(cfg: Dict[str, Any], shapes: Optional[Dict[str, Tuple[int, ...]]] = None, name: str = "Bedarax") -> HybridConfig:
+    """config.json of a Bedarax model -> HybridConfig.  `shapes` (tensor name -> shape, from the checkpoint's header) gives the
+    sizes config.json leaves to the tensors: the inner sizes of a channel_delta layer's two-step projections."""
+    shapes = shapes or {}
+    layers: List[LayerSpec] = []
+    for i, entry in enumerate(cfg["layers"]):
+        m, kind = entry["mixer"], entry["type"]
+        ff = _ff_spec(i, entry.get("mlp"))
+        H, G = int(m["heads"]), int(m.get("kv_heads", m["heads"]))
+        if H % G:
+            raise ValueError(f"layer {i}: {H} heads over {G} key heads")
+        if kind == "attention":
+            layers.append(LayerSpec(kind="attention", heads=H, kv_heads=G, dim=int(m["dim"]), vdim=int(m["vdim"]),
+                                    scale=float(m["scale"]), window=int((m.get("mask") or {}).get("size", 0)),
+                                    v_mix=bool(m.get("v_mix", False)), mlp=ff))
+        elif kind in ("delta", "channel_delta"):
+            d = int(m["dim"])
+            ra = rg = 0
+            if kind == "channel_delta":
+                ra = int(shapes.get(f"l{i}.mix.a1", (max(d // 2, 8),))[0])
+                rg = int(shapes.get(f"l{i}.mix.g1", (max(d // 2, 8),))[0])
+            layers.append(LayerSpec(kind=kind, heads=H, kv_heads=G, dim=d, vdim=int(m["vdim"]), conv=int(m.get("conv", 1)),
+                                    decay_rank=ra, gate_rank=rg, mlp=ff))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+    mixing = [s for s in layers if s.kind == "attention" and s.v_mix]
+    if any((s.kv_heads, s.vdim) != (mixing[0].kv_heads, mixing[0].vdim) for s in mixing):
+        raise ValueError("value-mixing attention layers must agree in key heads and value size")
+    return HybridConfig(vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]), layers=tuple(layers),
+                        rms_norm_eps=float(cfg["norm"]["eps"]), name=name, residual="pre_norm_depth")
+
+
 def rotary_table(spec: LayerSpec, max_position: int, device) -> torch.Tensor:
     """fp32 [max_position, rot_dims] = cos | sin of the layer's (scaled) rotary angles, amplitude folded in."""
     sc = dict(spec.rot_scaling) if spec.rot_scaling else None
@@ -123,7 +204,7 @@ def rotary_table(spec: LayerSpec, max_position: int, device) -> torch.Tensor:
 
 class _Layer:
     __slots__ = ("spec", "w_in", "o", "norm1", "norm2", "uk_t", "uv", "c_norm", "cos_sin", "out_norm", "decay", "router",
-                 "bias", "up", "down")
+                 "bias", "up", "down", "talk", "lam", "taps", "rate", "dt_bias", "a2", "g2", "act", "depth_w")
 
     def __init__(self, spec: LayerSpec) -> None:
         self.spec = spec
@@ -150,6 +231,8 @@ class HybridDecoder:
             return (torch.randn(shape, generator=g, device=device, dtype=torch.float32) * std).to(dtype)
 
         W = cfg.hidden_size
+        self.pre_norm = cfg.residual == "pre_norm_depth"
+        self.embed_norm = self.head = None
         self.embed = w(cfg.vocab_size, W, std=1.0)
         self.final_norm = w(W, std=0.1)
         self.layers: List[_Layer] = []
@@ -169,26 +252,63 @@ class HybridDecoder:
                 if key not in tables:
                     tables[key] = rotary_table(spec, self.max_position, device)
                 L.cos_sin = tables[key]
-            else:
+            elif spec.kind == "lightning":
                 L.w_in = w(2 * H * d + 2 * H * dv, W, std=W ** -0.5)  # q | k | v | gate
                 L.o = w(W, H * dv, std=(H * dv) ** -0.5)
                 L.out_norm = (1.0 + w(H * dv, std=0.1).float()).to(dtype)
                 L.decay = torch.tensor(spec.decay, dtype=torch.float32, device=device)
-            if spec.mlp is not None:
-                m = spec.mlp
+            elif spec.kind == "attention":
+                G = spec.kv_heads
+                L.w_in = w(H * d + G * d + G * dv + H, W, std=W ** -0.5)  # q | k | v | one gate per head
+                L.o = w(W, H * dv, std=(H * dv) ** -0.5)
+                L.talk = torch.eye(H, dtype=torch.float32, device=device) + w(H, H, std=0.2).float()
+                L.lam = w(1, std=0.3)
+            else:  # delta, channel_delta
+                G, C = spec.kv_heads, 2 * spec.kv_heads * d + H * dv
+                tail = spec.decay_rank + spec.gate_rank if spec.kind == "channel_delta" else H + H * dv
+                L.w_in = w(C + H + tail, W, std=W ** -0.5)  # q | k | v | beta | decay input | gate input
+                L.taps = w(C, spec.conv, std=spec.conv ** -0.5)
+                n_decay = H * d if spec.kind == "channel_delta" else H
+                L.rate = -torch.exp(w(H, std=0.5).float())  # -exp(A_log)
+                L.dt_bias = w(n_decay, std=0.5).float()
+                if spec.kind == "channel_delta":
+                    L.a2 = w(H * d, spec.decay_rank, std=spec.decay_rank ** -0.5)
+                    L.g2 = w(H * dv, spec.gate_rank, std=spec.gate_rank ** -0.5)
+                L.out_norm = (1.0 + w(dv, std=0.1).float()).to(dtype)
+                L.o = w(W, H * dv, std=(H * dv) ** -0.5)
+            m = spec.mlp
+            if isinstance(m, MoeSpec):
                 L.norm2 = w(W, std=0.1)
                 L.router = w(m.experts, W, std=W ** -0.5)
                 L.bias = w(m.experts, std=0.01)
-                L.up = w(m.experts, m.ff, W, std=W ** -0.5)
+                L.up = w(m.experts, (2 if m.gated else 1) * m.ff, W, std=W ** -0.5)  # gated: every expert's gate rows, then its up rows
                 L.down = w(m.experts, W, m.ff, std=m.ff ** -0.5)
+            elif isinstance(m, DenseFfSpec):
+                L.norm2 = w(W, std=0.1)
+                L.up = w(m.ff, W, std=W ** -0.5)
+                L.down = w(W, m.ff, std=m.ff ** -0.5)
+                L.act = torch.tensor([1.0, 0.3, 0.1, 0.01], dtype=torch.float32, device=device)
+            if self.pre_norm:
+                L.norm1, L.norm2 = (1.0 + L.norm1.float()).to(dtype), None if L.norm2 is None else (1.0 + L.norm2.float()).to(dtype)
+                c = torch.full((len(self.layers) + 2,), 0.1, dtype=torch.float32, device=device)
+                c[-1] = 1.0
+                L.depth_w = c
             self.layers.append(L)
+        if self.pre_norm:
+            self.final_norm = (1.0 + self.final_norm.float()).to(dtype)
+            self.embed_norm = (1.0 + w(W, std=0.1).float()).to(dtype)
+            self.head = w(cfg.vocab_size, W, std=W ** -0.5)
 
     # ------------------------------------------------------------------ weights
     def _tensors(self):
         yield self.embed
         yield self.final_norm
+        for t in (self.embed_norm, self.head):
+            if t is not None:
+                yield t
         for L in self.layers:
-            for k in ("w_in", "o", "norm1", "norm2", "uk_t", "uv", "c_norm", "out_norm", "router", "bias", "up", "down"):
+            for k in ("w_in", "o", "norm1", "norm2", "uk_t", "uv", "c_norm", "out_norm", "router", "bias", "up", "down", "talk", "lam",
+                      "taps", "rate", "dt_bias", "a2", "g2", "act", "depth_w"):
                 t = getattr(L, k)
                 if t is not None:
                     yield t
@@ -208,15 +328,34 @@ class HybridDecoder:
         def put(dst: torch.Tensor, src: torch.Tensor) -> None:
             if tuple(dst.shape) != tuple(src.shape):
                 raise ValueError(f"checkpoint tensor of shape {tuple(src.shape)} where the config implies {tuple(dst.shape)}")
-            dst.copy_(src.to(device=self.device, dtype=torch.float32).to(self.dtype))
+            dst.copy_(src.to(device=self.device, dtype=torch.float32))  # rounds to the destination's dtype (fp32 tensors stay fp32)
 
         put(self.embed, state["embed"])
         put(self.final_norm, state["final.norm"])
+        if self.pre_norm:
+            put(self.embed_norm, state["embed.norm"])
+            put(self.head, state["head"])
         for i, L in enumerate(self.layers):
             s, p = L.spec, f"l{i}.mix."
             H, d, dv = s.heads, s.dim, s.vdim
             put(L.norm1, state[f"l{i}.norm1"])
-            if s.kind == "latent_attention":
+            if L.depth_w is not None:
+                put(L.depth_w, state[f"l{i}.dwa"])
+            if s.kind == "attention":
+                put(L.w_in, torch.cat([state[p + "q"], state[p + "k"], state[p + "v"], state[p + "g"]], dim=0))
+                put(L.talk, state[p + "talk"])
+                put(L.lam, state[p + "vmix"].reshape(1) if (p + "vmix") in state else torch.zeros(1))
+            elif s.kind in ("delta", "channel_delta"):
+                tail = [state[p + "a1"], state[p + "g1"]] if s.kind == "channel_delta" else [state[p + "a"], state[p + "g"]]
+                put(L.w_in, torch.cat([state[p + "q"], state[p + "k"], state[p + "v"], state[p + "b"]] + tail, dim=0))
+                put(L.taps, torch.cat([state[p + "q.conv"], state[p + "k.conv"], state[p + "v.conv"]], dim=0))
+                put(L.rate, -torch.exp(state[p + "A_log"].to(torch.float32)))
+                put(L.dt_bias, state[p + "dt_bias"])
+                put(L.out_norm, state[p + "norm"])
+                if s.kind == "channel_delta":
+                    put(L.a2, state[p + "a2"])
+                    put(L.g2, state[p + "g2"])
+            elif s.kind == "latent_attention":
                 parts = [state[p + "q"]] + ([] if s.kv_from is not None else [state[p + "dkv"]])
                 put(L.w_in, torch.cat(parts, dim=0))
                 put(L.uk_t, state[p + "uk"].view(H, d, s.kv_rank).transpose(1, 2).contiguous())
@@ -227,10 +366,23 @@ class HybridDecoder:
                 put(L.w_in, torch.cat([state[p + "q"], state[p + "k"], state[p + "v"], state[p + "g"]], dim=0))
                 put(L.out_norm, state[p + "norm"])
             put(L.o, state[p + "o"])
-            if s.mlp is None and f"l{i}.norm2" in state:  # a layer without feed-forward that still norms a second time
+            if s.mlp is None and f"l{i}.norm2" in state and not self.pre_norm:  # no feed-forward, but a second norm all the same
                 L.norm2 = torch.empty_like(L.norm1)
                 put(L.norm2, state[f"l{i}.norm2"])
-            if s.mlp is not None:
+            if isinstance(s.mlp, DenseFfSpec):
+                q = f"l{i}.mlp."
+                put(L.norm2, state[f"l{i}.norm2"])
+                put(L.up, state[q + "up"])
+                put(L.down, state[q + "down"])
+                put(L.act, state[q + "act"])
+            elif isinstance(s.mlp, MoeSpec) and s.mlp.gated:
+                q = f"l{i}.mlp."
+                put(L.norm2, state[f"l{i}.norm2"])
+                put(L.router, state[q + "router"])
+                put(L.bias, state[q + "router.b"])
+                put(L.up, torch.stack([torch.cat([state[f"{q}e{e}.gate"], state[f"{q}e{e}.up"]], dim=0) for e in range(s.mlp.experts)]))
+                put(L.down, torch.stack([state[f"{q}e{e}.down"] for e in range(s.mlp.experts)]))
+            elif s.mlp is not None:
                 q = f"l{i}.mlp."
                 put(L.norm2, state[f"l{i}.norm2"])
                 put(L.router, state[q + "router"])
@@ -244,11 +396,29 @@ class HybridDecoder:
     def export_state(self) -> Dict[str, torch.Tensor]:
         """The inverse of load_state (checkpoint names, host tensors): what tests and tools hand to an independent implementation."""
         out = {"embed": self.embed, "final.norm": self.final_norm}
+        if self.pre_norm:
+            out["embed.norm"], out["head"] = self.embed_norm, self.head
         for i, L in enumerate(self.layers):
             s, p = L.spec, f"l{i}.mix."
             H, d, dv = s.heads, s.dim, s.vdim
             out[f"l{i}.norm1"] = L.norm1
-            if s.kind == "latent_attention":
+            if L.depth_w is not None:
+                out[f"l{i}.dwa"] = L.depth_w
+            if s.kind == "attention":
+                cuts = [H * d, s.kv_heads * d, s.kv_heads * dv, H]
+                out[p + "q"], out[p + "k"], out[p + "v"], out[p + "g"] = torch.split(L.w_in, cuts, dim=0)
+                out[p + "talk"], out[p + "vmix"] = L.talk, L.lam.reshape(())
+            elif s.kind in ("delta", "channel_delta"):
+                G, ch = s.kv_heads, s.kind == "channel_delta"
+                cuts = [G * d, G * d, H * dv, H] + ([s.decay_rank, s.gate_rank] if ch else [H, H * dv])
+                names = ["q", "k", "v", "b"] + (["a1", "g1"] if ch else ["a", "g"])
+                for n, t in zip(names, torch.split(L.w_in, cuts, dim=0)):
+                    out[p + n] = t
+                out[p + "q.conv"], out[p + "k.conv"], out[p + "v.conv"] = torch.split(L.taps, cuts[:3], dim=0)
+                out[p + "A_log"], out[p + "dt_bias"], out[p + "norm"] = torch.log(-L.rate), L.dt_bias, L.out_norm
+                if ch:
+                    out[p + "a2"], out[p + "g2"] = L.a2, L.g2
+            elif s.kind == "latent_attention":
                 nq = H * (d + s.rot_dim)
                 out[p + "q"] = L.w_in[:nq]
                 if s.kv_from is None:
@@ -262,7 +432,15 @@ class HybridDecoder:
             out[p + "o"] = L.o
             if s.mlp is None and L.norm2 is not None:
                 out[f"l{i}.norm2"] = L.norm2
-            if s.mlp is not None:
+            if isinstance(s.mlp, DenseFfSpec):
+                q = f"l{i}.mlp."
+                out[f"l{i}.norm2"], out[q + "up"], out[q + "down"], out[q + "act"] = L.norm2, L.up, L.down, L.act
+            elif isinstance(s.mlp, MoeSpec) and s.mlp.gated:
+                q = f"l{i}.mlp."
+                out[f"l{i}.norm2"], out[q + "router"], out[q + "router.b"] = L.norm2, L.router, L.bias
+                for e in range(s.mlp.experts):
+                    out[f"{q}e{e}.gate"], out[f"{q}e{e}.up"], out[f"{q}e{e}.down"] = L.up[e, : s.mlp.ff], L.up[e, s.mlp.ff:], L.down[e]
+            elif s.mlp is not None:
                 q = f"l{i}.mlp."
                 out[f"l{i}.norm2"], out[q + "router"] = L.norm2, L.router
                 if L.bias is not None:
@@ -317,11 +495,114 @@ class HybridDecoder:
         mixops.gemm_nt(y, act, L.down, n, W, m.ff, lda=m.ff, ldb=m.ff, ldc=W, groups=m.experts, b_gs=W * m.ff, seg=seg, c_rows=perm)
         return y
 
+    def _attention(self, i: int, L: _Layer, h: torch.Tensor, ctx: Any, batch: Any, shared: Dict[str, Any]) -> torch.Tensor:
+        """Windowed attention with mixed heads: projections, cache rows (values blended with the first value-mixing layer's),
+        scores / softmax / gate in one launch, output projection."""
+        s, md, kv = L.spec, batch.attn_metadata, ctx.kv_cache
+        T, H, G, d, dv = h.shape[0], s.heads, s.kv_heads, s.dim, s.vdim
+        proj = mixops.linear(h, L.w_in)
+        k_off, v_off, g_off = H * d, H * d + G * d, H * d + G * d + G * dv
+        first = shared.get("v_first") if s.v_mix else None
+        kc, vc = kv.kv_rows(i)
+        mixops.kv_store(kc, vc, batch.out_loc, proj, k_off, v_off, v_first=first, lam=L.lam if first is not None else None)
+        if s.v_mix and first is None:
+            shared["v_first"] = proj[:, v_off: v_off + G * dv]
+        o = torch.empty((T, H * dv), dtype=self.dtype, device=h.device)
+        mixops.window_attn(o, proj, g_off, kc, vc, ctx.page_table, md.req_rows, md.seq_lens, md.cu_seqlens_q, md.batch, H, G, d, dv,
+                           s.window, s.scale, L.talk)
+        return mixops.linear(o, L.o)
+
+    def _delta(self, i: int, L: _Layer, h: torch.Tensor, ctx: Any, batch: Any) -> torch.Tensor:
+        """Gated delta rule: projections, short convolution (+ unit vectors) with the request's conv state, the recurrence on
+        the request's fp32 state, per-head gated norm, output projection."""
+        s, md, kv = L.spec, batch.attn_metadata, ctx.kv_cache
+        T, H, G, d, dv = h.shape[0], s.heads, s.kv_heads, s.dim, s.vdim
+        C = 2 * G * d + H * dv
+        proj = mixops.linear(h, L.w_in)
+        qkv = mixops.short_conv(proj, C, L.taps, kv.conv_state(i), md.cu_seqlens_q, md.seq_lens, md.req_rows, md.batch,
+                                unit_heads=2 * G, scaled_heads=G, d=d)
+        b_raw = proj[:, C: C + H]
+        if s.kind == "channel_delta":
+            a_raw = mixops.linear(proj[:, C + H: C + H + s.decay_rank], L.a2)
+            gate = mixops.linear(proj[:, C + H + s.decay_rank: C + H + s.decay_rank + s.gate_rank], L.g2)
+            act = mixops.GATE_SIGMOID
+        else:
+            a_raw, gate, act = proj[:, C + H: C + 2 * H], proj[:, C + 2 * H: C + 2 * H + H * dv], mixops.GATE_SILU
+        o = torch.empty((T, H * dv), dtype=torch.float32, device=h.device)
+        mixops.delta_rule(o, qkv, kv.state(i), b_raw, a_raw, s.kind == "channel_delta", L.rate, L.dt_bias, md.cu_seqlens_q, md.seq_lens,
+                          md.req_rows, md.batch, G)
+        return mixops.linear(mixops.head_gated_norm(o, gate, L.out_norm, self.cfg.rms_norm_eps, H, dv, act), L.o)
+
+    def _gated_experts(self, L: _Layer, h: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+        """-> per-choice outputs [T, top, W] of experts W_down (silu(W_gate h) * (W_up h)); the weighted sum is the caller's."""
+        m, (T, W) = L.spec.mlp, h.shape
+        seg, perm = mixops.moe_sort(ids, m.experts)
+        n = T * m.top
+        gu = torch.empty((n, 2 * m.ff), dtype=self.dtype, device=h.device)
+        mixops.gemm_nt(gu, h, L.up, n, 2 * m.ff, W, lda=W, ldb=W, ldc=2 * m.ff, groups=m.experts, b_gs=2 * m.ff * W, seg=seg,
+                       a_rows=perm, a_div=m.top)
+        act = mixops.silu_mul(gu)
+        y = torch.empty((T, m.top, W), dtype=self.dtype, device=h.device)
+        mixops.gemm_nt(y, act, L.down, n, W, m.ff, lda=m.ff, ldb=m.ff, ldc=W, groups=m.experts, b_gs=W * m.ff, seg=seg, c_rows=perm)
+        return y
+
+    def _forward_pre_norm(self, ctx: Any, batch: Any, layer_outputs: Optional[list]) -> torch.Tensor:
+        """The pre-norm, depth-averaged stream -> the final-normed rows [tokens, W] in the model dtype."""
+        cfg, eps = self.cfg, self.cfg.rms_norm_eps
+        T, W, n = batch.input_ids.shape[0], cfg.hidden_size, len(self.layers)
+        dev = self.device
+        hist = torch.empty((n + 1, T, W), dtype=torch.float32, device=dev)  # X_0 .. X_n: what every layer's average reads
+        mixops.embed_norm(self.embed, batch.input_ids, self.embed_norm, eps, hist[0])
+        x = hist[0]
+        h = torch.empty((T, W), dtype=self.dtype, device=dev)
+        mid = torch.empty((T, W), dtype=torch.float32, device=dev)
+        mixops.prenorm(x, weight=self.layers[0].norm1 if n else self.final_norm, h_out=h, eps=eps)
+        shared: Dict[str, Any] = {}
+        for i, L in enumerate(self.layers):
+            kind, m = L.spec.kind, L.spec.mlp
+            if kind == "attention":
+                y = self._attention(i, L, h, ctx, batch, shared)
+            elif kind in ("delta", "channel_delta"):
+                y = self._delta(i, L, h, ctx, batch)
+            else:
+                raise NotImplementedError(f"mixer {kind!r} in a pre-norm stack")
+            nxt = self.layers[i + 1].norm1 if i + 1 < n else self.final_norm
+            x_next = torch.empty((T, W), dtype=torch.float32, device=dev)
+            if m is None:
+                mixops.prenorm(x, y=y, sum_out=hist[i + 1], history=hist, depth_w=L.depth_w, x_out=x_next, weight=nxt, h_out=h, eps=eps)
+            else:
+                if isinstance(m, DenseFfSpec):
+                    mixops.prenorm(x, y=y, sum_out=mid, weight=L.norm2, h_out=h, eps=eps)
+                    f, gate = mixops.linear(mixops.poly_act(mixops.linear(h, L.up), L.act, eps), L.down), None
+                else:
+                    fuse = T <= self.ROUTE_FUSE_MAX_TOKENS
+                    picks = mixops.prenorm(x, y=y, sum_out=mid, weight=L.norm2, h_out=h, eps=eps,
+                                           route=(L.router, L.bias, m.top) if fuse else None)
+                    if not fuse:
+                        picks = mixops.route_top(h, L.router, L.bias, m.top)
+                    f, gate = self._gated_experts(L, h, picks[0]), picks[1]
+                mixops.prenorm(mid, y=f, gate=gate, sum_out=hist[i + 1], history=hist, depth_w=L.depth_w, x_out=x_next, weight=nxt,
+                               h_out=h, eps=eps)
+            x = x_next
+            if layer_outputs is not None:
+                layer_outputs.append(x.clone())
+        return h
+
     def forward(self, ctx: Any, batch: Any, logits_out: Optional[torch.Tensor] = None, layer_outputs: Optional[list] = None) -> torch.Tensor:
         """-> logits [rows, vocab] in the model dtype: at `batch.logit_rows` (token indices) when set, else at every request's
         last token (prefill) or at every token (decode)."""
         cfg = self.cfg
         eps, alpha = cfg.rms_norm_eps, cfg.postln_alpha
+        if self.pre_norm:
+            hf = self._forward_pre_norm(ctx, batch, layer_outputs)
+            rows = getattr(batch, "logit_rows", None)
+            if rows is None and batch.is_prefill:
+                rows = batch.attn_metadata.get_last_indices(batch.size)
+            if rows is not None:
+                hf = hf.index_select(0, rows.to(torch.int64))
+            if logits_out is not None and logits_out.shape == (hf.shape[0], cfg.vocab_size) and logits_out.dtype == self.dtype:
+                return mixops.linear(hf, self.head, out=logits_out)
+            return mixops.linear(hf, self.head)
         x, h = mixops.embed(self.embed, batch.input_ids)
         for i, L in enumerate(self.layers):
             y = self._latent(i, L, h, ctx, batch) if L.spec.kind == "latent_attention" else self._lightning(i, L, h, ctx, batch)

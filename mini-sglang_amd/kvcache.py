@@ -96,11 +96,16 @@ class HybridCache:
     * a linear-recurrence layer keeps one fp32 state `[heads, dim, vdim]` per running request: `state(layer)` is
       `[state_rows, heads, dim, vdim]`, indexed by the request's page-table row, so a row that is handed to a new request
       brings its state slot with it (the kernel starts a request whose first token is at position 0 from zero).
+    * a key/value attention layer (`attention`) caches per token its keys `[kv_heads * dim]` and its (blended) values
+      `[kv_heads * vdim]` in the model dtype: `kv_rows(layer)` = two tensors indexed by the same token slots;
+    * a delta-rule layer (`delta`, `channel_delta`) keeps the fp32 state `[heads, dim, vdim]` like a lightning layer and,
+      beside it, the last `conv - 1` inputs of its short convolution: `conv_state(layer)` is `[state_rows, conv - 1,
+      channels]` in the model dtype, channels = 2 * kv_heads * dim + heads * vdim, same row index.
     Layers may differ in every size, so each gets its own allocation.
     """
 
     def __init__(self, layers, num_pages: int, page_size: int, state_rows: int, dtype: torch.dtype, device: torch.device) -> None:
-        self._latent, self._state, self._owner = {}, {}, {}
+        self._latent, self._state, self._owner, self._kv, self._conv = {}, {}, {}, {}, {}
         slots = num_pages * page_size
         for i, spec in enumerate(layers):
             if spec.kind == "latent_attention":
@@ -109,6 +114,16 @@ class HybridCache:
                 self._owner[i] = i if spec.kv_from is None else spec.kv_from
             elif spec.kind == "lightning":
                 self._state[i] = torch.zeros((state_rows, spec.heads, spec.dim, spec.vdim), dtype=torch.float32, device=device)
+            elif spec.kind == "attention":
+                self._kv[i] = (torch.zeros((slots, spec.kv_heads * spec.dim), dtype=dtype, device=device),
+                               torch.zeros((slots, spec.kv_heads * spec.vdim), dtype=dtype, device=device))
+            elif spec.kind in ("delta", "channel_delta"):
+                self._state[i] = torch.zeros((state_rows, spec.heads, spec.dim, spec.vdim), dtype=torch.float32, device=device)
+                if spec.conv > 1:
+                    channels = 2 * spec.kv_heads * spec.dim + spec.heads * spec.vdim
+                    self._conv[i] = torch.zeros((state_rows, spec.conv - 1, channels), dtype=dtype, device=device)
+            else:
+                raise ValueError(f"layer {i}: no cache layout for mixer {spec.kind!r}")
         for i, j in self._owner.items():
             if j not in self._latent:
                 raise ValueError(f"layer {i} borrows the keys of layer {j}, which caches none")
@@ -123,14 +138,27 @@ class HybridCache:
     def state(self, layer: int) -> torch.Tensor:
         return self._state[layer]
 
+    def kv_rows(self, layer: int):
+        """(keys [slots, kv_heads * dim], values [slots, kv_heads * vdim]) of a key/value attention layer."""
+        return self._kv[layer]
+
+    def conv_state(self, layer: int):
+        """[state_rows, conv - 1, channels] of a delta-rule layer, or None when its convolution has one tap."""
+        return self._conv.get(layer)
+
     @staticmethod
     def bytes_per_page(layers, page_size: int, dtype: torch.dtype) -> int:
         es = torch.empty((), dtype=dtype).element_size()
-        return sum((s.kv_rank + s.rot_dim) * es * page_size for s in layers if s.kind == "latent_attention" and s.kv_from is None)
+        per_token = sum(s.kv_rank + s.rot_dim for s in layers if s.kind == "latent_attention" and s.kv_from is None)
+        per_token += sum(s.kv_heads * (s.dim + s.vdim) for s in layers if s.kind == "attention")
+        return per_token * es * page_size
 
     @staticmethod
-    def state_bytes(layers, state_rows: int) -> int:
-        return sum(4 * s.heads * s.dim * s.vdim * state_rows for s in layers if s.kind == "lightning")
+    def state_bytes(layers, state_rows: int, dtype: torch.dtype = torch.bfloat16) -> int:
+        es = torch.empty((), dtype=dtype).element_size()
+        total = sum(4 * s.heads * s.dim * s.vdim * state_rows for s in layers if s.kind in ("lightning", "delta", "channel_delta"))
+        return total + sum(es * (s.conv - 1) * (2 * s.kv_heads * s.dim + s.heads * s.vdim) * state_rows
+                           for s in layers if s.kind in ("delta", "channel_delta"))
 
     @property
     def device(self) -> torch.device:

@@ -1,4 +1,4 @@
-"""torch-facing wrappers of the sequence-mixing kernels (include/msgl_mix.h, csrc/seqmix.hip).
+"""torch-facing wrappers of the sequence-mixing kernels (include/msgl_mix.h, csrc/seqmix.hip, csrc/mix_delta.hip).
 
 Same rules as ops.py: device tensors only, no CPU fallback, pointers + sizes + the current stream go straight to
 the C ABI.  `linear` is the projection seam of the hybrid models: the library GEMM (bf16, or fp32 in the library's
@@ -232,4 +232,184 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None)
         except _lib.MsglError:
             _NO_LIBRARY_SOLUTION.add(key)
     gemm_nt(out, x, w, M, N, K, lda=x.stride(0), ldb=w.stride(0), ldc=out.stride(0))
+    return out
+
+
+# ------------------------------------------------------------------ pre-norm hybrid decoders (csrc/mix_delta.hip)
+GATE_SIGMOID, GATE_SILU = 0, 1
+
+
+def embed_norm(table: torch.Tensor, ids: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> torch.Tensor:
+    """out (fp32 [T, W]) = the embedding rows divided by their root mean square, times `weight`."""
+    _dev(table, ids, weight, out)
+    T, W = ids.shape[0], table.shape[1]
+    assert table.is_contiguous() and weight.dtype == table.dtype and weight.shape == (W,) and weight.is_contiguous()
+    assert out.dtype == torch.float32 and out.is_contiguous() and out.shape == (T, W)
+    check_mix(mix_lib().msgl_mix_embed_norm(out.data_ptr(), table.data_ptr(), _i32(ids).data_ptr(), weight.data_ptr(), float(eps), T, W,
+                                            _code(table), _stream()), "embed_norm")
+    return out
+
+
+def prenorm(x: torch.Tensor, *, y: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+            sum_out: Optional[torch.Tensor] = None, history: Optional[torch.Tensor] = None, depth_w: Optional[torch.Tensor] = None,
+            x_out: Optional[torch.Tensor] = None, weight: Optional[torch.Tensor] = None, h_out: Optional[torch.Tensor] = None,
+            eps: float = 1e-6, route=None, dtype: Optional[torch.dtype] = None):
+    """s = x + sum_p gate[:, p] y[:, p] -> sum_out;  with depth_w (fp32 [n]) the row that goes on is
+    sum_{j < n - 1} depth_w[j] history[j] + depth_w[n - 1] s -> x_out (history: fp32 [>= n - 1, rows, W]; sum_out may be
+    history[n - 1]);  weight: h_out = rms_unit(row) * weight in the weight's dtype.  route = (router [E, W], bias [E] | None, top):
+    the normed rows are routed in the same launch -> (expert ids int32 [rows, top], softmax weights fp32 [rows, top])."""
+    _dev(x, y, gate, sum_out, history, depth_w, x_out, weight, h_out)
+    rows, W = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    parts = 0
+    if y is not None:
+        assert y.is_contiguous() and y.shape[0] == rows and y.shape[-1] == W
+        parts = 1 if y.dim() == 2 else y.shape[1]
+    t = weight if weight is not None else y
+    assert t is not None and (y is None or weight is None or y.dtype == weight.dtype)
+    if gate is not None:
+        assert gate.dtype == torch.float32 and gate.is_contiguous() and gate.numel() == rows * parts
+    for o in (sum_out, x_out):
+        assert o is None or (o.shape == (rows, W) and o.is_contiguous() and o.dtype == torch.float32)
+    n_mix = 0
+    if depth_w is not None:
+        n_mix = depth_w.numel()
+        assert depth_w.dtype == torch.float32 and depth_w.is_contiguous() and x_out is not None
+        assert n_mix == 1 or (history is not None and history.dtype == torch.float32 and history.is_contiguous()
+                              and history.shape[0] >= n_mix - 1 and history.shape[1:] == (rows, W))
+    if weight is not None:
+        assert weight.shape == (W,) and weight.is_contiguous() and h_out is not None
+        assert h_out.shape == (rows, W) and h_out.is_contiguous() and h_out.dtype == weight.dtype
+    router = bias = ids = wts = None
+    E = top = 0
+    if route is not None:
+        router, bias, top = route
+        _dev(router, bias)
+        E = router.shape[0]
+        assert router.shape == (E, W) and router.is_contiguous() and router.dtype == weight.dtype
+        assert bias is None or (bias.dtype == weight.dtype and bias.shape == (E,) and bias.is_contiguous())
+        ids = torch.empty((rows, top), dtype=torch.int32, device=x.device)
+        wts = torch.empty((rows, top), dtype=torch.float32, device=x.device)
+    if rows:
+        check_mix(mix_lib().msgl_mix_prenorm(
+            x.data_ptr(), _p(y), parts, _p(gate), _p(sum_out), _p(history), 0 if history is None else history.stride(0), _p(depth_w),
+            n_mix, _p(x_out), _p(weight), _p(h_out), float(eps), rows, W, _code(t), _p(router), _p(bias), E, top, _p(ids), _p(wts),
+            _stream()), "prenorm")
+    return None if route is None else (ids, wts)
+
+
+def poly_act(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """coef[0] N(z) + coef[1] N(z^2) + coef[2] N(z^3) + coef[3] per row (N = divide by the row's root mean square)."""
+    _dev(z, coef)
+    rows, N = z.shape
+    assert z.stride(1) == 1 and coef.dtype == torch.float32 and coef.numel() == 4 and coef.is_contiguous()
+    out = torch.empty((rows, N), dtype=z.dtype, device=z.device)
+    check_mix(mix_lib().msgl_mix_poly_act(out.data_ptr(), z.data_ptr(), z.stride(0), coef.data_ptr(), float(eps), rows, N, _code(z),
+                                          _stream()), "poly_act")
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """rows [gate | up] of 2 N -> silu(gate) * up, rows of N."""
+    _dev(gate_up)
+    rows, N2 = gate_up.shape
+    assert gate_up.is_contiguous() and N2 % 2 == 0
+    out = torch.empty((rows, N2 // 2), dtype=gate_up.dtype, device=gate_up.device)
+    check_mix(mix_lib().msgl_mix_silu_mul(out.data_ptr(), gate_up.data_ptr(), rows, N2 // 2, _code(gate_up), _stream()), "silu_mul")
+    return out
+
+
+def route_top(h: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+    """-> (expert ids int32 [T, top], weights fp32 [T, top]): fp32 logits (product kernel, fp32 accumulation) + bias, the `top`
+    largest win, weights = softmax over the winners."""
+    _dev(h, router, bias)
+    T, W = h.shape
+    E = router.shape[0]
+    assert h.is_contiguous() and router.is_contiguous() and router.shape == (E, W) and router.dtype == h.dtype
+    assert bias is None or (bias.dtype == h.dtype and bias.shape == (E,) and bias.is_contiguous())
+    z = torch.empty((T, E), dtype=torch.float32, device=h.device)
+    gemm_nt(z, h, router, T, E, W, lda=W, ldb=W, ldc=E)
+    ids = torch.empty((T, top), dtype=torch.int32, device=h.device)
+    wts = torch.empty((T, top), dtype=torch.float32, device=h.device)
+    check_mix(mix_lib().msgl_mix_route_top(ids.data_ptr(), wts.data_ptr(), z.data_ptr(), _p(bias), T, E, top, _code(h), _stream()),
+              "route_top")
+    return ids, wts
+
+
+def kv_store(k_cache: torch.Tensor, v_cache: torch.Tensor, out_loc: torch.Tensor, src: torch.Tensor, k_off: int, v_off: int,
+             v_first: Optional[torch.Tensor] = None, lam: Optional[torch.Tensor] = None) -> None:
+    """k = src[:, k_off : +nk], v = src[:, v_off : +nv] -> the cache rows at out_loc; v blended with v_first by `lam` when given."""
+    _dev(k_cache, v_cache, out_loc, src, v_first, lam)
+    T = src.shape[0]
+    nk, nv = k_cache.shape[1], v_cache.shape[1]
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == src.dtype == v_cache.dtype
+    assert src.stride(1) == 1 and out_loc.shape[0] == T
+    if v_first is not None:
+        assert v_first.dtype == src.dtype and v_first.stride(1) == 1 and v_first.shape == (T, nv) and lam.dtype == src.dtype
+    check_mix(mix_lib().msgl_mix_kv_store(
+        k_cache.data_ptr(), v_cache.data_ptr(), _i32(out_loc).data_ptr(), src.data_ptr(), src.stride(0), k_off, v_off, nk, nv,
+        _p(v_first), 0 if v_first is None else v_first.stride(0), _p(lam), T, _code(src), _stream()), "kv_store")
+
+
+def window_attn(out: torch.Tensor, src: torch.Tensor, g_off: int, k_cache: torch.Tensor, v_cache: torch.Tensor, table: torch.Tensor,
+                req_rows: torch.Tensor, seq_lens: torch.Tensor, cu_q: torch.Tensor, batch: int, H: int, G: int, d: int, dv: int,
+                window: int, scale: float, talk: torch.Tensor) -> None:
+    """Sliding-window attention with the heads' scores mixed by `talk` (fp32 [H, H]) and a sigmoid gate per head (src[:, g_off + h]);
+    q = src[:, : H * d].  out: [T, H * dv] in the model dtype."""
+    _dev(out, src, k_cache, v_cache, table, req_rows, seq_lens, cu_q, talk)
+    T = src.shape[0]
+    assert src.stride(1) == 1 and out.is_contiguous() and out.shape == (T, H * dv) and out.dtype == src.dtype
+    assert k_cache.is_contiguous() and k_cache.shape[1] == G * d and v_cache.is_contiguous() and v_cache.shape[1] == G * dv
+    assert k_cache.dtype == src.dtype == v_cache.dtype and talk.dtype == torch.float32 and talk.is_contiguous() and talk.shape == (H, H)
+    assert table.dtype == torch.int32 and table.stride(1) == 1
+    assert req_rows.numel() >= batch and seq_lens.numel() >= batch and cu_q.numel() >= batch + 1
+    check_mix(mix_lib().msgl_mix_window_attn(
+        out.data_ptr(), src.data_ptr(), src.stride(0), g_off, k_cache.data_ptr(), v_cache.data_ptr(), table.data_ptr(), table.stride(0),
+        _i32(req_rows).data_ptr(), _i32(seq_lens).data_ptr(), _i32(cu_q).data_ptr(), batch, T, H, G, d, dv, window, float(scale),
+        talk.data_ptr(), _code(src), _stream()), "window_attn")
+
+
+def short_conv(src: torch.Tensor, C: int, taps: torch.Tensor, state: Optional[torch.Tensor], cu_q: torch.Tensor, seq_lens: torch.Tensor,
+               slots: torch.Tensor, batch: int, unit_heads: int, scaled_heads: int, d: int) -> torch.Tensor:
+    """Causal per-channel convolution + SiLU of src[:, :C] (taps [C, n]; state [slots, n - 1, C] carries the inputs before the
+    portion and is moved on), unit vectors for the first `unit_heads` groups of d channels -> fp32 [T, C]."""
+    _dev(src, taps, state, cu_q, seq_lens, slots)
+    T, n = src.shape[0], taps.shape[1]
+    assert src.stride(1) == 1 and taps.is_contiguous() and taps.shape[0] == C and taps.dtype == src.dtype
+    assert n == 1 or (state.is_contiguous() and state.dtype == src.dtype and state.shape[1:] == (n - 1, C))
+    out = torch.empty((T, C), dtype=torch.float32, device=src.device)
+    check_mix(mix_lib().msgl_mix_short_conv(
+        out.data_ptr(), src.data_ptr(), src.stride(0), taps.data_ptr(), _p(state), _i32(cu_q).data_ptr(), _i32(seq_lens).data_ptr(),
+        _i32(slots).data_ptr(), batch, T, C, n, unit_heads, scaled_heads, d, _code(src), _stream()), "short_conv")
+    return out
+
+
+def delta_rule(out: torch.Tensor, qkv: torch.Tensor, state: torch.Tensor, b_raw: torch.Tensor, a_raw: torch.Tensor, per_channel: bool,
+               rate: torch.Tensor, dt_bias: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor, slots: torch.Tensor, batch: int,
+               G: int) -> None:
+    """state: fp32 [slots, H, d, dv]; qkv: fp32 rows [q G*d | k G*d | v H*dv]; b_raw [T, H], a_raw [T, H] or [T, H*d] in the model
+    dtype (views with a row stride are fine); rate = -exp(A_log) and dt_bias in fp32."""
+    _dev(out, qkv, state, b_raw, a_raw, rate, dt_bias, cu_q, seq_lens, slots)
+    _, H, d, dv = state.shape
+    T = qkv.shape[0]
+    na = H * d if per_channel else H
+    assert state.dtype == torch.float32 and state.is_contiguous() and qkv.dtype == torch.float32 and qkv.is_contiguous()
+    assert qkv.shape == (T, 2 * G * d + H * dv) and out.dtype == torch.float32 and out.is_contiguous() and out.shape == (T, H * dv)
+    assert b_raw.stride(1) == 1 and a_raw.stride(1) == 1 and b_raw.shape == (T, H) and a_raw.shape == (T, na) and a_raw.dtype == b_raw.dtype
+    assert rate.dtype == torch.float32 and rate.shape == (H,) and dt_bias.dtype == torch.float32 and dt_bias.shape == (na,)
+    check_mix(mix_lib().msgl_mix_delta_rule(
+        out.data_ptr(), qkv.data_ptr(), state.data_ptr(), b_raw.data_ptr(), b_raw.stride(0), a_raw.data_ptr(), a_raw.stride(0),
+        int(per_channel), rate.data_ptr(), dt_bias.data_ptr(), _i32(cu_q).data_ptr(), _i32(seq_lens).data_ptr(), _i32(slots).data_ptr(),
+        batch, H, G, d, dv, _code(b_raw), _stream()), "delta_rule")
+
+
+def head_gated_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, H: int, dv: int, gate_act: int) -> torch.Tensor:
+    """Per head: o / rms(o) * weight[dv] * act(gate) -> [rows, H * dv] in the gate's dtype."""
+    _dev(o, gate, weight)
+    rows = o.shape[0]
+    assert o.dtype == torch.float32 and o.is_contiguous() and o.shape == (rows, H * dv) and gate.shape == (rows, H * dv)
+    assert gate.stride(1) == 1 and weight.dtype == gate.dtype and weight.shape == (dv,) and weight.is_contiguous()
+    out = torch.empty((rows, H * dv), dtype=gate.dtype, device=o.device)
+    check_mix(mix_lib().msgl_mix_head_gated_norm(out.data_ptr(), o.data_ptr(), gate.data_ptr(), gate.stride(0), weight.data_ptr(),
+                                                 float(eps), rows, H, dv, gate_act, _code(gate), _stream()), "head_gated_norm")
     return out

@@ -10,7 +10,7 @@ import json
 from pathlib import Path
 from typing import Any, Callable, Dict, Tuple
 
-from .hybrid import HybridConfig, HybridDecoder
+from .hybrid import HybridConfig, HybridDecoder, bedarax_config
 from .model import DenseDecoder, ModelConfig
 
 
@@ -38,6 +38,7 @@ def _load_hybrid(model: HybridDecoder, state: Dict[str, Any]) -> None:
 # name in config.json -> (configuration reader, decoder class, weight loader)
 ARCHITECTURES: Dict[str, Tuple[Callable[[Dict[str, Any]], Any], type, Callable[[Any, Dict[str, Any]], None]]] = {
     "Nidorax": (HybridConfig.from_json, HybridDecoder, _load_hybrid),
+    "Bedarax": (bedarax_config, HybridDecoder, _load_hybrid),
     "Qwen3ForCausalLM": (dense_config_from_hf, DenseDecoder, _load_dense),
     "Qwen2ForCausalLM": (dense_config_from_hf, DenseDecoder, _load_dense),
     "LlamaForCausalLM": (dense_config_from_hf, DenseDecoder, _load_dense),
@@ -58,12 +59,30 @@ def model_class(cfg: Any) -> type:
     return HybridDecoder if isinstance(cfg, HybridConfig) else DenseDecoder
 
 
+def checkpoint_shapes(path) -> Dict[str, Tuple[int, ...]]:
+    """Tensor name -> shape from the header of the folder's model.safetensors (8-byte little-endian length, then that many
+    bytes of JSON); {} when there is no such file.  No tensor data is read."""
+    file = Path(path) / "model.safetensors"
+    if not file.exists():
+        return {}
+    with open(file, "rb") as f:
+        n = int.from_bytes(f.read(8), "little")
+        header = json.loads(f.read(n))
+    return {k: tuple(v["shape"]) for k, v in header.items() if k != "__metadata__"}
+
+
 def load_model_dir(path) -> Tuple[Any, str]:
-    """-> (configuration object, registered architecture name) of the folder's config.json."""
+    """-> (configuration object, registered architecture name) of the folder's config.json.  A reader that declares a `shapes`
+    parameter also gets the checkpoint's tensor shapes: some designs leave sizes to them."""
+    import inspect
+
     with open(Path(path) / "config.json") as f:
         raw = json.load(f)
     name = architecture_of(raw)
-    return ARCHITECTURES[name][0](raw), name
+    reader = ARCHITECTURES[name][0]
+    if "shapes" in inspect.signature(reader).parameters:
+        return reader(raw, shapes=checkpoint_shapes(path)), name
+    return reader(raw), name
 
 
 def load_weights(model: Any, path, name: str) -> None:
