@@ -666,7 +666,17 @@ def main() -> None:
                          "lightning recurrence + routed experts) beside a dense decoder of equal size, and its kernels against "
                          "their rooflines (tools/hybrid_bench.py; further flags after --hybrid-args)")
     ap.add_argument("--hybrid-args", nargs=argparse.REMAINDER, default=[], help="flags handed to tools/hybrid_bench.py")
+    ap.add_argument("--bedarax", action="store_true",
+                    help="instead of the default workload: prefill / decode throughput of the pre-norm hybrid decoder (windowed "
+                         "attention with mixed heads + gated delta-rule layers) beside the post-norm hybrid decoder of equal size, "
+                         "and its kernels against their rooflines (tools/bedarax_bench.py; further flags after --bedarax-args)")
+    ap.add_argument("--bedarax-args", nargs=argparse.REMAINDER, default=[], help="flags handed to tools/bedarax_bench.py")
     args = ap.parse_args()
+    if args.bedarax:
+        from tools.bedarax_bench import main as bedarax_main
+
+        bedarax_main(list(args.bedarax_args))
+        return
     if args.hybrid:
         from tools.hybrid_bench import main as hybrid_main
 

@@ -129,10 +129,14 @@ int msgl_mix_kv_store(void* k_cache, void* v_cache, const int* out_loc, const vo
 /* Causal attention over the last `window` keys (0 = all) with the heads' scores mixed before the softmax:
  * s_h(i, j) = scale * sum_g talk[h, g] q_g(i) . k_group(g)(j), softmax over visible j in fp32, o_h = sum_j p_h(j) v_group(h)(j),
  * out[t, h] = o_h * sigmoid(src[t, g_off + h]) in T.  q = src[t, 0 : H d]; cache rows [slots, G d] / [slots, G dv]; requests as in
- * msgl_mix_latent_attn (table rows of token slots, seq_lens = keys after this forward, cu_q = prefix of new tokens). */
+ * msgl_mix_latent_attn (table rows of token slots, seq_lens = keys after this forward, cu_q = prefix of new tokens).
+ * `splits` > 1 cuts every token's visible keys into that many ranges whose partial results (workspace: fp32,
+ * msgl_mix_window_attn_workspace_floats) a second launch merges -- for steps with few query tokens. */
+int msgl_mix_window_attn_workspace_floats(int total_q, int H, int dv, int splits);
 int msgl_mix_window_attn(void* out, const void* src, int64_t ld_src, int g_off, const void* k_cache, const void* v_cache, const int* table,
                          int64_t table_stride, const int* req_rows, const int* seq_lens, const int* cu_q, int batch, int total_q, int H,
-                         int G, int d, int dv, int window, float scale, const float* talk, int dtype, void* stream);
+                         int G, int d, int dv, int window, float scale, const float* talk, int dtype, int splits, float* workspace,
+                         void* stream);
 
 /* Causal convolution over time per channel, then SiLU: out[t, c] = silu(sum_j taps[c, j] in[pos - (n - 1) + j, c]) (fp32);
  * inputs of this forward are src[t, 0 : C], earlier ones come from state[slots[b]] ([n - 1, C] in T per request: the inputs

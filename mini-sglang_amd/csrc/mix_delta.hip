@@ -206,111 +206,223 @@ __global__ __launch_bounds__(256) void kv_store_kernel(T* __restrict__ k_cache, 
 }
 
 // ------------------------------------------------------------------------------------------------ windowed attention with mixed heads
-// One workgroup (256 threads) per query token, all H heads.  Keys j with max(0, p - window + 1) <= j <= p in tiles of 64:
-//   raw[g][key] = q_g . k_{group(g)}[key]          thread = (key, every fourth head)
-//   s[h][key]   = scale * sum_g talk[h][g] raw[g][key]
-//   online softmax per head (a wave takes every fourth head, lane = key), p -> LDS
-//   acc[h][e]  = acc * corr[h] + sum_key p[h][key] v_{group(h)}[key][e]       thread = output element (h, e)
-// out[t, h, e] = acc / l[h] * sigmoid(gate[t, h]) in T.
+// One workgroup (256 threads) = QT consecutive query tokens of one request x all H heads (x one of `splits` ranges of the keys).
+// Keys from the first query's window start to the last query's position, in tiles of 64:
+//   raw[g][q][key] = q_g . k_{group(g)}[key]        thread = (key, every fourth head): a key row is loaded once for the QT queries
+//   s[h][q][key]   = scale * sum_g talk[h][g] raw[g][q][key], masked per query (causal, window)
+//   online softmax per (head, query) (a wave takes every fourth head, lane = key), p -> LDS
+//   acc[q][h][e]  = acc * corr + sum_key p[h][q][key] v_{group(h)}[key][e]    thread = (head, 8 consecutive e): 16-byte value loads
+// splits == 1: out[t, h, e] = acc / l * sigmoid(gate[t, h]) in T.  splits > 1: every range leaves (acc, m, l) in the workspace and
+// window_merge_kernel joins them -- for steps with few query tokens (decode), where one workgroup per token leaves the chip empty.
 constexpr int kAttnAcc = 16;  // H * dv <= 256 * kAttnAcc
 
-template <typename T>
-__global__ __launch_bounds__(256) void window_attn_kernel(T* __restrict__ out, const T* __restrict__ src, int64_t ld_src, int g_off,
+template <typename T, int QT>
+__global__ __launch_bounds__(256) void window_attn_kernel(T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+                                                          const T* __restrict__ src, int64_t ld_src, int g_off,
                                                           const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                                                           const int* __restrict__ table, int64_t table_stride,
                                                           const int* __restrict__ req_rows, const int* __restrict__ seq_lens,
-                                                          const int* __restrict__ cu_q, int batch, int H, int G, int d, int dv, int window,
-                                                          float scale, const float* __restrict__ talk) {
-  extern __shared__ float lds[];
-  float* q = lds;                       // H * d
-  float* tk = q + H * d;                // H * H
-  float* raw = tk + H * H;              // H * 64
-  float* pr = raw + H * 64;             // H * 64
-  float* mrow = pr + H * 64;            // H
-  float* lrow = mrow + H;               // H
-  float* corr = lrow + H;               // H
-  int* slots = reinterpret_cast<int*>(corr + H);  // 64
-  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int b = request_of(cu_q, batch, t);
-  const int n_new = cu_q[b + 1] - cu_q[b];
-  const int p = seq_lens[b] - n_new + (t - cu_q[b]);
-  const int j0 = window > 0 && p - window + 1 > 0 ? p - window + 1 : 0;
+                                                          const int* __restrict__ cu_q, int batch, int total_q, int H, int G, int d, int dv,
+                                                          int window, float scale, const float* __restrict__ talk, int splits) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* tk = lds;                       // H * H
+  float* raw = tk + H * H;               // H * QT * 64
+  float* pr = raw + H * QT * 64;         // H * QT * 64
+  float* mrow = pr + H * QT * 64;        // H * QT
+  float* lrow = mrow + H * QT;           // H * QT
+  float* corr = lrow + H * QT;           // H * QT
+  int* slots = reinterpret_cast<int*>(corr + H * QT);  // 64
+  T* qs = reinterpret_cast<T*>(lds + ((H * H + 2 * H * QT * 64 + 3 * H * QT + 64 + 3) & ~3));  // QT * H * d, 16-byte aligned
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // which request and which of its query tiles
+  int wg = blockIdx.x, b = 0, n_new = 0;
+  for (; b < batch; ++b) {
+    n_new = cu_q[b + 1] - cu_q[b];
+    const int nt = (n_new + QT - 1) / QT;
+    if (wg < nt) break;
+    wg -= nt;
+  }
+  if (b == batch) return;
+  const int q0 = wg * QT, nq = n_new - q0 < QT ? n_new - q0 : QT;
+  const int t0 = cu_q[b] + q0, p0 = seq_lens[b] - n_new + q0;
+  const int j_lo = window > 0 && p0 - window + 1 > 0 ? p0 - window + 1 : 0, j_hi = p0 + nq - 1;
+  const int ntiles = (j_hi - j_lo) / 64 + 1, per = (ntiles + splits - 1) / splits;
+  const int tile_lo = blockIdx.y * per, tile_hi = tile_lo + per < ntiles ? tile_lo + per : ntiles;
   const int* trow = table + (size_t)req_rows[b] * table_stride;
-  const T* qrow = src + (size_t)t * ld_src;
-  for (int i = tid; i < H * d; i += 256) q[i] = ld(qrow + i);
+  const int Hd = H * d;
+  for (int i = tid; i < nq * Hd; i += 256) qs[i] = src[(size_t)(t0 + i / Hd) * ld_src + i % Hd];
   for (int i = tid; i < H * H; i += 256) tk[i] = talk[i] * scale;
-  for (int i = tid; i < H; i += 256) {
+  for (int i = tid; i < H * QT; i += 256) {
     mrow[i] = -INFINITY;
     lrow[i] = 0.f;
   }
   const int rep = H / G, nk = G * d, nv = G * dv, no = H * dv;
-  float acc[kAttnAcc];
+  float acc[QT][kAttnAcc];
 #pragma unroll
-  for (int a = 0; a < kAttnAcc; ++a) acc[a] = 0.f;
-  const bool wide = (d & 7) == 0;
-  for (int base = j0; base <= p; base += 64) {
+  for (int qi = 0; qi < QT; ++qi)
+#pragma unroll
+    for (int a = 0; a < kAttnAcc; ++a) acc[qi][a] = 0.f;
+  const bool wide_k = (d & 7) == 0, wide_v = (dv & 7) == 0;
+  for (int tile = tile_lo; tile < tile_hi; ++tile) {
+    const int base = j_lo + tile * 64;
     __syncthreads();
-    if (tid < 64) slots[tid] = base + tid <= p ? trow[base + tid] : -1;
+    if (tid < 64) slots[tid] = base + tid <= j_hi ? trow[base + tid] : -1;
     __syncthreads();
-    const int slot = slots[lane];
+    const int slot = slots[lane], pos = base + lane;
     for (int g = wave; g < H; g += 4) {
-      float s = 0.f;
+      float s[QT];
+#pragma unroll
+      for (int qi = 0; qi < QT; ++qi) s[qi] = 0.f;
       if (slot >= 0) {
         const T* kr = k_cache + (size_t)slot * nk + (size_t)(g / rep) * d;
-        const float* qg = q + g * d;
-        if (wide) {
+        if (wide_k) {
           for (int i = 0; i < d; i += 8) {
             float kv[8];
             read8(kr + i, kv);
 #pragma unroll
-            for (int u = 0; u < 8; ++u) s = fmaf(qg[i + u], kv[u], s);
+            for (int qi = 0; qi < QT; ++qi) {
+              if (qi < nq) {
+                float qv[8];
+                read8(qs + qi * Hd + g * d + i, qv);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) s[qi] = fmaf(qv[u], kv[u], s[qi]);
+              }
+            }
           }
         } else {
-          for (int i = 0; i < d; ++i) s = fmaf(qg[i], ld(kr + i), s);
+          for (int i = 0; i < d; ++i) {
+            const float kv = ld(kr + i);
+#pragma unroll
+            for (int qi = 0; qi < QT; ++qi)
+              if (qi < nq) s[qi] = fmaf(ld(qs + qi * Hd + g * d + i), kv, s[qi]);
+          }
         }
       }
-      raw[g * 64 + lane] = s;
+#pragma unroll
+      for (int qi = 0; qi < QT; ++qi) raw[(g * QT + qi) * 64 + lane] = s[qi];
     }
     __syncthreads();
     for (int h = wave; h < H; h += 4) {
-      float s = 0.f;
-      for (int g = 0; g < H; ++g) s = fmaf(tk[h * H + g], raw[g * 64 + lane], s);
-      if (slot < 0) s = -INFINITY;
-      const float m_old = mrow[h];
-      const float m_new = fmaxf(m_old, wave_max(s));
-      const float pv = slot < 0 ? 0.f : expf(s - m_new);
-      const float sum = wave_sum(pv);
-      pr[h * 64 + lane] = pv;
-      if (lane == 0) {
-        const float cf = expf(m_old - m_new);
-        corr[h] = cf;
-        lrow[h] = lrow[h] * cf + sum;
-        mrow[h] = m_new;
+#pragma unroll
+      for (int qi = 0; qi < QT; ++qi) {
+        if (qi >= nq) break;
+        float s = 0.f;
+        for (int g = 0; g < H; ++g) s = fmaf(tk[h * H + g], raw[(g * QT + qi) * 64 + lane], s);
+        const int pq = p0 + qi;
+        const bool seen = slot >= 0 && pos <= pq && (window <= 0 || pq - pos < window);
+        if (!seen) s = -INFINITY;
+        const float m_old = mrow[h * QT + qi];
+        const float m_new = fmaxf(m_old, wave_max(s));
+        const float pv = seen ? expf(s - m_new) : 0.f;
+        const float sum = wave_sum(pv);
+        pr[(h * QT + qi) * 64 + lane] = pv;
+        if (lane == 0) {
+          const float cf = m_new == -INFINITY ? 1.f : expf(m_old - m_new);  // no key of this query so far: nothing to rescale
+          corr[h * QT + qi] = cf;
+          lrow[h * QT + qi] = lrow[h * QT + qi] * cf + sum;
+          mrow[h * QT + qi] = m_new;
+        }
       }
     }
     __syncthreads();
-    const int keys = p - base + 1 < 64 ? p - base + 1 : 64;
+    const int keys = j_hi - base + 1 < 64 ? j_hi - base + 1 : 64;
+    if (wide_v) {
+      const int per_head = dv >> 3;
 #pragma unroll
-    for (int a = 0; a < kAttnAcc; ++a) {
-      const int o = tid + 256 * a;
-      if (o < no) {
-        const int h = o / dv, e = o - h * dv;
-        const T* vcol = v_cache + (size_t)(h / rep) * dv + e;
-        const float* ph = pr + h * 64;
-        float s = acc[a] * corr[h];
-        for (int key = 0; key < keys; ++key) s = fmaf(ph[key], ld(vcol + (size_t)slots[key] * nv), s);
-        acc[a] = s;
+      for (int a = 0; a < kAttnAcc / 8; ++a) {
+        const int c = tid + 256 * a;
+        if (c < H * per_head) {
+          const int h = c / per_head, e0 = (c - h * per_head) << 3;
+          const T* vcol = v_cache + (size_t)(h / rep) * dv + e0;
+#pragma unroll
+          for (int qi = 0; qi < QT; ++qi) {
+            const float cf = corr[h * QT + qi];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc[qi][a * 8 + u] *= cf;
+          }
+          for (int key = 0; key < keys; ++key) {
+            float vv[8];
+            read8(vcol + (size_t)slots[key] * nv, vv);
+#pragma unroll
+            for (int qi = 0; qi < QT; ++qi) {
+              const float p = pr[(h * QT + qi) * 64 + key];
+#pragma unroll
+              for (int u = 0; u < 8; ++u) acc[qi][a * 8 + u] = fmaf(p, vv[u], acc[qi][a * 8 + u]);
+            }
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int a = 0; a < kAttnAcc; ++a) {
+        const int o = tid + 256 * a;
+        if (o < no) {
+          const int h = o / dv, e = o - h * dv;
+          const T* vcol = v_cache + (size_t)(h / rep) * dv + e;
+#pragma unroll
+          for (int qi = 0; qi < QT; ++qi) acc[qi][a] *= corr[h * QT + qi];
+          for (int key = 0; key < keys; ++key) {
+            const float vv = ld(vcol + (size_t)slots[key] * nv);
+#pragma unroll
+            for (int qi = 0; qi < QT; ++qi) acc[qi][a] = fmaf(pr[(h * QT + qi) * 64 + key], vv, acc[qi][a]);
+          }
+        }
       }
     }
   }
   __syncthreads();
+  // element o of a token's output row <-> (a, u) of this thread
+  const int per_head = dv >> 3;
 #pragma unroll
   for (int a = 0; a < kAttnAcc; ++a) {
-    const int o = tid + 256 * a;
-    if (o < no) {
-      const int h = o / dv;
-      st(out + (size_t)t * no + o, acc[a] / lrow[h] * sigmoidf_(ld(qrow + g_off + h)));
+    int o;
+    if (wide_v) {
+      const int c = tid + 256 * (a >> 3);
+      o = c < H * per_head ? c * 8 + (a & 7) : no;
+    } else {
+      o = tid + 256 * a;
     }
+    if (o >= no) continue;
+    const int h = o / dv;
+#pragma unroll
+    for (int qi = 0; qi < QT; ++qi) {
+      if (qi >= nq) break;
+      const size_t t = (size_t)(t0 + qi);
+      if (splits == 1)
+        st(out + t * no + o, acc[qi][a] / lrow[h * QT + qi] * sigmoidf_(ld(src + t * ld_src + g_off + h)));
+      else
+        part_o[((size_t)blockIdx.y * total_q + t) * no + o] = acc[qi][a];
+    }
+  }
+  if (splits > 1)
+    for (int i = tid; i < H * nq; i += 256) {
+      const int h = i / nq, qi = i - h * nq;
+      float* ml = part_ml + (((size_t)blockIdx.y * total_q + t0 + qi) * H + h) * 2;
+      ml[0] = mrow[h * QT + qi];
+      ml[1] = lrow[h * QT + qi];
+    }
+}
+
+// Joins the key ranges of window_attn_kernel: one workgroup per token.
+template <typename T>
+__global__ __launch_bounds__(256) void window_merge_kernel(T* __restrict__ out, const float* __restrict__ part_o,
+                                                           const float* __restrict__ part_ml, const T* __restrict__ src, int64_t ld_src,
+                                                           int g_off, int total_q, int H, int dv, int splits) {
+  const size_t t = blockIdx.x;
+  const int no = H * dv;
+  for (int o = threadIdx.x; o < no; o += 256) {
+    const int h = o / dv;
+    float m = -INFINITY;
+    for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(((size_t)s * total_q + t) * H + h) * 2]);
+    float l = 0.f, v = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float* ml = part_ml + (((size_t)s * total_q + t) * H + h) * 2;
+      if (ml[0] == -INFINITY) continue;
+      const float f = expf(ml[0] - m);
+      l = fmaf(ml[1], f, l);
+      v = fmaf(part_o[((size_t)s * total_q + t) * no + o], f, v);
+    }
+    st(out + t * no + o, v / l * sigmoidf_(ld(src + t * ld_src + g_off + h)));
   }
 }
 
@@ -555,24 +667,51 @@ int msgl_mix_kv_store(void* k_cache, void* v_cache, const int* out_loc, const vo
   return MSGL_MIX_OK;
 }
 
+int msgl_mix_window_attn_workspace_floats(int total_q, int H, int dv, int splits) {
+  return splits > 1 ? splits * total_q * (H * dv + 2 * H) : 0;
+}
+
 int msgl_mix_window_attn(void* out, const void* src, int64_t ld_src, int g_off, const void* k_cache, const void* v_cache, const int* table,
                          int64_t table_stride, const int* req_rows, const int* seq_lens, const int* cu_q, int batch, int total_q, int H,
-                         int G, int d, int dv, int window, float scale, const float* talk, int dtype, void* stream) {
+                         int G, int d, int dv, int window, float scale, const float* talk, int dtype, int splits, float* workspace,
+                         void* stream) {
   MIX_REQUIRE(out && src && k_cache && v_cache && table && req_rows && seq_lens && cu_q && talk && dtype_ok(dtype),
               "window_attn: null pointer / dtype");
   MIX_REQUIRE(batch >= 0 && total_q >= 0 && H >= 1 && G >= 1 && H % G == 0 && d >= 1 && dv >= 1 && window >= 0,
               "window_attn: bad sizes H %d G %d d %d dv %d window %d", H, G, d, dv, window);
   MIX_REQUIRE(H * dv <= 256 * kAttnAcc, "window_attn: %d output elements per token (at most %d)", H * dv, 256 * kAttnAcc);
   MIX_REQUIRE(ld_src >= (int64_t)H * d && ld_src >= g_off + H && g_off >= 0, "window_attn: columns past the source row");
-  MIX_REQUIRE(dtype == MSGL_MIX_F32 || (d % 8 != 0) || ((G * d) % 8 == 0), "window_attn: key rows not 16-byte aligned");
+  MIX_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || workspace), "window_attn: %d key ranges need a workspace", splits);
   if (total_q == 0 || batch == 0) return MSGL_MIX_OK;
-  const size_t lds = (size_t)(H * d + H * H + 2 * H * 64 + 3 * H + 64) * sizeof(float);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)window_attn_kernel<T>, lds) == 0, "window_attn: %zu bytes of LDS", lds);
-             hipLaunchKernelGGL(window_attn_kernel<T>, dim3(total_q), dim3(256), lds, s, mp<T>(out), cp<T>(src), ld_src, g_off,
-                                cp<T>(k_cache), cp<T>(v_cache), table, table_stride, req_rows, seq_lens, cu_q, batch, H, G, d, dv, window,
-                                scale, talk);)
+  const size_t es = dtype == MSGL_MIX_BF16 ? 2 : 4;
+  float* part_o = workspace;
+  float* part_ml = workspace ? workspace + (size_t)splits * total_q * H * dv : nullptr;
+  // query tokens per workgroup: 8 where portions are long and the tile fits half the LDS (two workgroups per CU), else 4, else 1
+#define WA_LAUNCH(QT)                                                                                                                  \
+  {                                                                                                                                    \
+    const size_t lds = (size_t)(H * H + 2 * H * QT * 64 + 3 * H * QT + 64 + 3) * sizeof(float) + (size_t)QT * H * d * es;                  \
+    const int tiles = total_q / QT + batch;                                                                                            \
+    DISPATCH_T(dtype, MIX_REQUIRE(ensure_lds((const void*)window_attn_kernel<T, QT>, lds) == 0, "window_attn: %zu bytes of LDS", lds); \
+               hipLaunchKernelGGL((window_attn_kernel<T, QT>), dim3(tiles, splits), dim3(256), lds, s, mp<T>(out), part_o, part_ml,     \
+                                  cp<T>(src), ld_src, g_off, cp<T>(k_cache), cp<T>(v_cache), table, table_stride, req_rows, seq_lens,  \
+                                  cu_q, batch, total_q, H, G, d, dv, window, scale, talk, splits);)                                     \
+  }
+  const auto lds_of = [&](int qt) { return (size_t)(H * H + 2 * H * qt * 64 + 3 * H * qt + 64 + 3) * 4 + (size_t)qt * H * d * es; };
+  if (total_q >= 8 * batch && lds_of(8) <= 80 * 1024) {
+    WA_LAUNCH(8)
+  } else if (total_q >= 4 * batch && lds_of(4) <= 80 * 1024) {
+    WA_LAUNCH(4)
+  } else {
+    WA_LAUNCH(1)
+  }
+#undef WA_LAUNCH
   MIX_LAUNCHED("window_attn");
+  if (splits > 1) {
+    DISPATCH_T(dtype, hipLaunchKernelGGL(window_merge_kernel<T>, dim3(total_q), dim3(256), 0, s, mp<T>(out), part_o, part_ml, cp<T>(src),
+                                         ld_src, g_off, total_q, H, dv, splits);)
+    MIX_LAUNCHED("window_attn (merge)");
+  }
   return MSGL_MIX_OK;
 }
 

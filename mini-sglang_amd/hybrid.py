@@ -509,7 +509,7 @@ class HybridDecoder:
             shared["v_first"] = proj[:, v_off: v_off + G * dv]
         o = torch.empty((T, H * dv), dtype=self.dtype, device=h.device)
         mixops.window_attn(o, proj, g_off, kc, vc, ctx.page_table, md.req_rows, md.seq_lens, md.cu_seqlens_q, md.batch, H, G, d, dv,
-                           s.window, s.scale, L.talk)
+                           s.window, s.scale, L.talk, splits=mixops.window_attn_splits(md.batch, T, s.window, md.max_seqlen_k))
         return mixops.linear(o, L.o)
 
     def _delta(self, i: int, L: _Layer, h: torch.Tensor, ctx: Any, batch: Any) -> torch.Tensor:

@@ -351,11 +351,21 @@ def kv_store(k_cache: torch.Tensor, v_cache: torch.Tensor, out_loc: torch.Tensor
         _p(v_first), 0 if v_first is None else v_first.stride(0), _p(lam), T, _code(src), _stream()), "kv_store")
 
 
+def window_attn_splits(batch: int, total_q: int, window: int, max_keys: int) -> int:
+    """Key ranges per token for a step with few query tokens: enough workgroups to fill the chip, at least two 64-key tiles each.
+    A function of static sizes only (rows, the window or the LONGEST possible key count), so a captured graph keeps its grid."""
+    if total_q >= 8 * batch and total_q >= 256:
+        return 1
+    keys = min(window, max_keys) if window > 0 else max_keys
+    return max(1, min(512 // max(total_q, 1), keys // 128, 32))
+
+
 def window_attn(out: torch.Tensor, src: torch.Tensor, g_off: int, k_cache: torch.Tensor, v_cache: torch.Tensor, table: torch.Tensor,
                 req_rows: torch.Tensor, seq_lens: torch.Tensor, cu_q: torch.Tensor, batch: int, H: int, G: int, d: int, dv: int,
-                window: int, scale: float, talk: torch.Tensor) -> None:
+                window: int, scale: float, talk: torch.Tensor, splits: int = 1) -> None:
     """Sliding-window attention with the heads' scores mixed by `talk` (fp32 [H, H]) and a sigmoid gate per head (src[:, g_off + h]);
-    q = src[:, : H * d].  out: [T, H * dv] in the model dtype."""
+    q = src[:, : H * d].  out: [T, H * dv] in the model dtype.  splits > 1: the visible keys of every token in that many ranges
+    (partial results merged by a second launch), for steps with few query tokens."""
     _dev(out, src, k_cache, v_cache, table, req_rows, seq_lens, cu_q, talk)
     T = src.shape[0]
     assert src.stride(1) == 1 and out.is_contiguous() and out.shape == (T, H * dv) and out.dtype == src.dtype
@@ -363,10 +373,13 @@ def window_attn(out: torch.Tensor, src: torch.Tensor, g_off: int, k_cache: torch
     assert k_cache.dtype == src.dtype == v_cache.dtype and talk.dtype == torch.float32 and talk.is_contiguous() and talk.shape == (H, H)
     assert table.dtype == torch.int32 and table.stride(1) == 1
     assert req_rows.numel() >= batch and seq_lens.numel() >= batch and cu_q.numel() >= batch + 1
+    ws = None
+    if splits > 1:
+        ws = torch.empty(mix_lib().msgl_mix_window_attn_workspace_floats(T, H, dv, splits), dtype=torch.float32, device=out.device)
     check_mix(mix_lib().msgl_mix_window_attn(
         out.data_ptr(), src.data_ptr(), src.stride(0), g_off, k_cache.data_ptr(), v_cache.data_ptr(), table.data_ptr(), table.stride(0),
         _i32(req_rows).data_ptr(), _i32(seq_lens).data_ptr(), _i32(cu_q).data_ptr(), batch, T, H, G, d, dv, window, float(scale),
-        talk.data_ptr(), _code(src), _stream()), "window_attn")
+        talk.data_ptr(), _code(src), splits, _p(ws), _stream()), "window_attn")
 
 
 def short_conv(src: torch.Tensor, C: int, taps: torch.Tensor, state: Optional[torch.Tensor], cu_q: torch.Tensor, seq_lens: torch.Tensor,

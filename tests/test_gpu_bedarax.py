@@ -151,11 +151,13 @@ def _window_reference(q, k, v, gate, talk, scale, window, rep):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("splits", [1, 3], ids=["one-range", "three-ranges"])
 @pytest.mark.parametrize("window", [1, 5, 16, 17, 63, 64, 65, 130, 0])
-def test_window_edges_one_key_stands_out(dev, dtype, window):
+def test_window_edges_one_key_stands_out(dev, dtype, window, splits):
     """One loud key: every query that still sees it must put (nearly) all its weight there, the first query past the window
     none.  The sequence is cut into a prompt portion and single decoded tokens, its slots are scattered over the pool, and the
-    loud key sits so that its last visible query falls once in the portion and once among the decoded tokens."""
+    loud key sits so that its last visible query falls once in the portion and once among the decoded tokens; with the keys
+    of every token in one range and cut into three (partial results merged)."""
     from mini_sglang_amd import mixops
 
     H, G, d, dv, scale = 4, 2, 16, 24, 0.5
@@ -188,7 +190,7 @@ def test_window_edges_one_key_stands_out(dev, dtype, window):
             part = torch.empty((hi - lo, H * dv), dtype=dtype, device=dev)
             mixops.window_attn(part, src[lo:hi], H * d, kc, vc, table.to(dev), torch.tensor([2], dtype=torch.int32, device=dev),
                                torch.tensor([hi], dtype=torch.int32, device=dev), torch.tensor([0, hi - lo], dtype=torch.int32, device=dev),
-                               1, H, G, d, dv, window, scale, talk.float().to(dev))
+                               1, H, G, d, dv, window, scale, talk.float().to(dev), splits=splits)
             got[lo:hi] = part
         got = got.double().cpu().view(T, H, dv)
         tol = 1e-5 if dtype == torch.float32 else 2e-2
