@@ -151,10 +151,15 @@ int msgl_mix_short_conv(float* out, const void* src, int64_t ld_src, const void*
  * [q: G x d | k: G x d | v: H x dv] (head h reads q/k group h / (H / G)); state: fp32 [slots, H, d, dv], row slots[b], zero for a
  * request whose first new token is at position 0; beta = sigmoid(b_raw[t, h]); g = exp(rate[h] * softplus(a_raw[t, i] +
  * dt_bias[i])) with i = h (per_channel = 0: one decay per head) or h * d + channel (per_channel = 1: one per row of S);
- * rate = -exp(A_log) in fp32.  out: fp32 [tokens, H * dv]. */
+ * rate = -exp(A_log) in fp32.  out: fp32 [tokens, H * dv].
+ * n_items > 0: the new tokens are cut into chunks that run in parallel (items / item_first as in msgl_mix_lightning).  The rule is
+ * linear in S, so a chunk is S_end = P S_start + L: one launch computes every chunk's (L | P) by running the rule over dv + d
+ * columns from (0 | identity), a scan walks each request's chunks, a third launch computes every chunk's outputs from its start
+ * state.  scratch: fp32, n_items * H * d * (2 dv + d) floats. */
 int msgl_mix_delta_rule(float* out, const float* qkv, float* state, const void* b_raw, int64_t ld_b, const void* a_raw, int64_t ld_a,
                         int per_channel, const float* rate, const float* dt_bias, const int* cu_q, const int* seq_lens, const int* slots,
-                        int batch, int H, int G, int d, int dv, int dtype, void* stream);
+                        int batch, int H, int G, int d, int dv, int dtype, int n_items, const int* items, const int* item_first,
+                        float* scratch, void* stream);
 
 /* out[t, h, e] = o[t, h, e] / sqrt(mean_e(o[t, h]^2) + eps) * w[e] * act(gate[t, h * dv + e]); act: 0 = sigmoid, 1 = SiLU. */
 int msgl_mix_head_gated_norm(void* out, const float* o, const void* gate, int64_t ld_gate, const void* w, float eps, int rows, int H,

@@ -162,7 +162,7 @@ MIX_SIGNATURES = {
     "msgl_mix_window_attn_workspace_floats": (_i, [_i, _i, _i, _i]),
     "msgl_mix_window_attn": (_i, [_p, _p, _l, _i, _p, _p, _p, _l, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p, _i, _i, _p, _p]),
     "msgl_mix_short_conv": (_i, [_p, _p, _l, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p]),
-    "msgl_mix_delta_rule": (_i, [_p, _p, _p, _p, _l, _p, _l, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
+    "msgl_mix_delta_rule": (_i, [_p, _p, _p, _p, _l, _p, _l, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p]),
     "msgl_mix_head_gated_norm": (_i, [_p, _p, _p, _l, _p, _f, _i, _i, _i, _i, _i, _p]),
 }
 

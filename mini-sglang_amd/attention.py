@@ -36,6 +36,7 @@ class HipAttnMetadata:
     tile_order: Optional[torch.Tensor] = None  # [total_tiles] int32: q tiles, most keys first (prefill only)
     plan: Optional[torch.Tensor] = None     # decode work list (device)
     chunks: Optional[tuple] = None          # recurrent layers: (items [n, 3], item_first [B + 1], n) of long portions cut in pieces
+    delta_chunks: Optional[tuple] = None    # the same list at the delta-rule layers' piece size
 
     def get_last_indices(self, bs: int) -> torch.Tensor:
         return self.cu_seqlens_q[1: 1 + bs] - 1
@@ -222,6 +223,7 @@ class MixAttnBackend:
     as the request's state slot.  Graph capture keeps static copies of the vectors, refreshed before every replay."""
 
     RECURRENT_CHUNK = 128
+    DELTA_CHUNK = 256
 
     def __init__(self, config: Any, ctx: Any = None, *, tp_size: int = 1) -> None:
         ctx = ctx if ctx is not None else _core.get_global_ctx()
@@ -231,6 +233,7 @@ class MixAttnBackend:
         self.max_bs = int(ctx.page_table.shape[0])
         self.capture_bs: List[int] = []
         self._cap: Optional[torch.Tensor] = None
+        self._kinds = {getattr(s, "kind", "") for s in getattr(config, "layers", ())}
 
     def prepare_metadata(self, batch: Any) -> None:
         reqs = batch.padded_reqs
@@ -238,26 +241,36 @@ class MixAttnBackend:
         q = np.fromiter((r.extend_len for r in reqs), dtype=np.int64, count=bs)
         k = np.fromiter((r.device_len for r in reqs), dtype=np.int64, count=bs)
         rows = np.fromiter((r.table_idx for r in reqs), dtype=np.int64, count=bs)
-        # a long portion's recurrence runs as pieces of RECURRENT_CHUNK tokens in parallel (their states joined by a scan)
-        pieces = -(-q // self.RECURRENT_CHUNK)
-        n_items = int(pieces.sum()) if int(q.max()) >= 2 * self.RECURRENT_CHUNK else 0
-        host = torch.empty(3 * bs + 1 + (3 * n_items + bs + 1 if n_items else 0), dtype=torch.int32, pin_memory=True)
+        # a long portion's recurrence runs as pieces in parallel (their states joined by a scan): RECURRENT_CHUNK tokens for the
+        # decay-only recurrence, DELTA_CHUNK for the delta rule, whose scan step is a [d, d] x [d, dv] product per piece
+        lists = []
+        if int(q.max()) >= 2 * self.RECURRENT_CHUNK and self._kinds & {"lightning"}:
+            lists.append(("chunks", self.RECURRENT_CHUNK))
+        if int(q.max()) >= 2 * self.DELTA_CHUNK and self._kinds & {"delta", "channel_delta"}:
+            lists.append(("delta_chunks", self.DELTA_CHUNK))
+        pieces = [-(-q // c) for _, c in lists]
+        extra = sum(3 * int(p.sum()) + bs + 1 for p in pieces)
+        host = torch.empty(3 * bs + 1 + extra, dtype=torch.int32, pin_memory=True)
         h = host.numpy()
         h[:bs], h[bs: 2 * bs], h[2 * bs] = k, rows, 0
         h[2 * bs + 1: 3 * bs + 1] = np.cumsum(q)
-        if n_items:
-            req = np.repeat(np.arange(bs), pieces)
-            first = np.cumsum(pieces) - pieces
-            begin = (np.arange(n_items) - first[req]) * self.RECURRENT_CHUNK
-            items = h[3 * bs + 1: 3 * bs + 1 + 3 * n_items].reshape(n_items, 3)
-            items[:, 0], items[:, 1], items[:, 2] = req, begin, np.minimum(begin + self.RECURRENT_CHUNK, q[req])
-            h[3 * bs + 1 + 3 * n_items] = 0
-            h[3 * bs + 2 + 3 * n_items:] = np.cumsum(pieces)
+        at, where = 3 * bs + 1, []
+        for (name, c), p in zip(lists, pieces):
+            n_items = int(p.sum())
+            req = np.repeat(np.arange(bs), p)
+            first = np.cumsum(p) - p
+            begin = (np.arange(n_items) - first[req]) * c
+            items = h[at: at + 3 * n_items].reshape(n_items, 3)
+            items[:, 0], items[:, 1], items[:, 2] = req, begin, np.minimum(begin + c, q[req])
+            h[at + 3 * n_items] = 0
+            h[at + 3 * n_items + 1: at + 3 * n_items + bs + 1] = np.cumsum(p)
+            where.append((name, at, n_items))
+            at += 3 * n_items + bs + 1
         dev = host.to(self.device, non_blocking=True)
         batch.attn_metadata = HipAttnMetadata(cu_seqlens_q=dev[2 * bs: 3 * bs + 1], seq_lens=dev[:bs], req_rows=dev[bs: 2 * bs], batch=bs,
                                               max_seqlen_q=int(q.max()), max_seqlen_k=int(k.max()))
-        if n_items:
-            batch.attn_metadata.chunks = (dev[3 * bs + 1: 3 * bs + 1 + 3 * n_items], dev[3 * bs + 1 + 3 * n_items:], n_items)
+        for name, at, n_items in where:
+            setattr(batch.attn_metadata, name, (dev[at: at + 3 * n_items], dev[at + 3 * n_items: at + 3 * n_items + bs + 1], n_items))
 
     # ------------------------------------------------------------------ graph hooks
     def init_capture_graph(self, max_seq_len: int, bs_list: List[int]) -> None:

@@ -19,7 +19,8 @@
 //   short_conv_kernel        causal per-channel convolution over time + SiLU, inputs before the portion from the request's
 //                            conv state; q / k heads made unit vectors (q also * d^-1/2);  conv_state_kernel shifts the state
 //   delta_rule_kernel        S <- decay S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q   per (request, head); a thread
-//                            owns one value column of S in registers; scalar or per-key-channel decay
+//                            owns one value column of S in registers; scalar or per-key-channel decay; long portions as
+//                            parallel chunks: per-chunk transition (L | P), delta_scan_kernel over a request's chunks, outputs
 //   head_gated_norm_kernel   per-head rms over dv * w * (sigmoid | silu)(gate)
 #include "mix_common.h"
 
@@ -485,36 +486,79 @@ __global__ __launch_bounds__(256) void conv_state_kernel(T* __restrict__ state, 
 }
 
 // ------------------------------------------------------------------------------------------------ gated delta rule
-// Workgroup = (column block of 64, head, request); a thread owns column e of the head's state S [d, dv] (DP >= d registers, the
-// tail zero).  Per token, with g the decay (one number per head, or one per key channel = row of S):
+// Workgroup = (column block of 64, head, request or chunk); a thread owns column e of the head's state S [d, dv] (DP >= d
+// registers, the tail zero).  Per token, with g the decay (one number per head, or one per key channel = row of S):
 //   S <- g S;  u = beta (v_e - S^T k);  S <- S + k u;  o_e = S^T q
-// computed as  dk = S_old . (g k), dq = S_old . (g q), u = beta (v_e - dk), S = g S_old + k u, o_e = dq + u (k . q):  the same
-// numbers, one pass less over the column.  q, k (fp32, unit vectors) come from qkv rows [q: G x d | k: G x d | v: H x dv];
-// beta = sigmoid(b_raw[t, h]);  g = exp(rate[h] * softplus(a_raw[t, .] + dt_bias[.])) with rate = -exp(A_log) (fp32, from the host).
-// 16 tokens (8 for the widest heads) are staged in LDS at a time.  A request whose portion starts at position 0 starts from S = 0.
-template <typename T, int DP, bool CHANNEL>
+// computed as  dk = S_old . (g k), u = beta (v_e - dk), S = g S_old + k u, o_e = S . q  (two passes over the column).  q, k (fp32,
+// unit vectors) come from qkv rows [q: G x d | k: G x d | v: H x dv]; beta = sigmoid(b_raw[t, h]);
+// g = exp(rate[h] * softplus(a_raw[t, .] + dt_bias[.])) with rate = -exp(A_log) (fp32, from the host).  16 tokens (8 for the
+// widest heads) are staged in LDS at a time: k, g k, g, q per key channel, the block's 64 values, beta.
+//
+// MODE 0  a request's whole portion from its state row (zero when the portion starts at position 0), state row written back.
+// Long portions are cut into chunks that run in parallel.  The rule is linear in S: over a chunk S_end = P S_start + L with
+// P [d, d] the product of the tokens' transitions and L [d, dv] the state the chunk builds from zero.
+// MODE 1  a chunk's (L | P): the same recurrence over dv + d columns, values = (v | 0), start = (0 | identity), no outputs;
+//         -> scratch[item][h][d][dv + d].  The last chunk of a request is skipped (nothing follows it).
+//         delta_scan_kernel then walks a request's chunks: start[c + 1] = P_c start[c] + L_c.
+// MODE 2  a chunk's outputs from its start state; the last chunk of a request writes the state row.
+template <typename T, int DP, bool CHANNEL, int MODE>
 __global__ __launch_bounds__(64) void delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qkv, float* __restrict__ state,
                                                         const T* __restrict__ b_raw, int64_t ld_b, const T* __restrict__ a_raw,
                                                         int64_t ld_a, const float* __restrict__ rate, const float* __restrict__ dt_bias,
                                                         const int* __restrict__ cu_q, const int* __restrict__ seq_lens,
-                                                        const int* __restrict__ slots, int H, int G, int d, int dv) {
+                                                        const int* __restrict__ slots, int H, int G, int d, int dv,
+                                                        const int* __restrict__ items, const int* __restrict__ item_first,
+                                                        float* __restrict__ scratch, float* __restrict__ start) {
   constexpr int kStage = DP > 128 ? 8 : 16;
-  __shared__ __attribute__((aligned(16))) float sk[kStage][DP], sgk[kStage][DP], sgq[kStage][DP], sg[kStage][DP];
-  __shared__ float skq[kStage], sbeta[kStage];
-  const int b = blockIdx.z, h = blockIdx.y, e = blockIdx.x * 64 + threadIdx.x, lane = threadIdx.x;
-  const int first = cu_q[b], n_new = cu_q[b + 1] - first;
+  __shared__ __attribute__((aligned(16))) float sk[kStage][DP], sgk[kStage][DP], sq[kStage][DP], sg[kStage][DP];
+  __shared__ float sv[kStage][64], sbeta[kStage], sdec[kStage];
+  const int h = blockIdx.y, e = blockIdx.x * 64 + threadIdx.x, lane = threadIdx.x;
+  int b, first, n_new;
+  bool last_chunk = true;
+  if (MODE == 0) {
+    b = blockIdx.z;
+    first = cu_q[b];
+    n_new = cu_q[b + 1] - first;
+  } else {
+    const int it = blockIdx.z;
+    b = items[3 * it];
+    first = cu_q[b] + items[3 * it + 1];
+    n_new = items[3 * it + 2] - items[3 * it + 1];
+    last_chunk = it == item_first[b + 1] - 1;
+    if (MODE == 1 && last_chunk) return;
+  }
   if (n_new <= 0) return;
-  const bool fresh = seq_lens[b] == n_new;
   const int C = 2 * G * d + H * dv, kvh = h / (H / G);
-  float* Srow = state + ((size_t)slots[b] * H + h) * d * dv;
-  const bool live = e < dv;
+  const int cols = MODE == 1 ? dv + d : dv;
+  const bool live = e < cols, value_col = e < dv;
   float S[DP];
+  if (MODE == 0) {
+    const bool fresh = seq_lens[b] == n_new;
+    const float* Srow = state + ((size_t)slots[b] * H + h) * d * dv;
 #pragma unroll
-  for (int i = 0; i < DP; ++i) S[i] = (!fresh && live && i < d) ? Srow[(size_t)i * dv + e] : 0.f;
+    for (int i = 0; i < DP; ++i) S[i] = (!fresh && live && i < d) ? Srow[(size_t)i * dv + e] : 0.f;
+  } else if (MODE == 1) {
+#pragma unroll
+    for (int i = 0; i < DP; ++i) S[i] = (live && !value_col && i == e - dv) ? 1.f : 0.f;
+  } else {
+    const float* Srow = start + ((size_t)blockIdx.z * H + h) * d * dv;
+#pragma unroll
+    for (int i = 0; i < DP; ++i) S[i] = (live && i < d) ? Srow[(size_t)i * dv + e] : 0.f;
+  }
   const float r = rate[h];
   for (int t0 = 0; t0 < n_new; t0 += kStage) {
     const int nt = n_new - t0 < kStage ? n_new - t0 : kStage;
     __syncthreads();
+    if (lane < nt) {
+      const size_t t = (size_t)(first + t0 + lane);
+      sbeta[lane] = sigmoidf_(ld(b_raw + t * ld_b + h));
+      if (!CHANNEL) sdec[lane] = expf(r * softplusf_(ld(a_raw + t * ld_a + h) + dt_bias[h]));
+    }
+    for (int idx = lane; idx < nt * 64; idx += 64) {
+      const int tt = idx >> 6;
+      sv[tt][lane] = (live && value_col) ? qkv[(size_t)(first + t0 + tt) * C + 2 * G * d + h * dv + e] : 0.f;
+    }
+    if (!CHANNEL) __syncthreads();
     for (int idx = lane; idx < nt * DP; idx += 64) {
       const int tt = idx / DP, i = idx - tt * DP;
       const size_t t = (size_t)(first + t0 + tt);
@@ -522,41 +566,95 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(float* __restrict__ out,
       if (i < d) {
         qv = qkv[t * C + kvh * d + i];
         kv = qkv[t * C + (G + kvh) * d + i];
-        const int ai = CHANNEL ? h * d + i : h;
-        g = expf(r * softplusf_(ld(a_raw + t * ld_a + ai) + dt_bias[ai]));
+        g = CHANNEL ? expf(r * softplusf_(ld(a_raw + t * ld_a + h * d + i) + dt_bias[h * d + i])) : sdec[tt];
       }
       sk[tt][i] = kv;
       sgk[tt][i] = g * kv;
-      sgq[tt][i] = g * qv;
+      sq[tt][i] = qv;
       sg[tt][i] = g;
-    }
-    if (lane < nt) {
-      const size_t t = (size_t)(first + t0 + lane);
-      float kq = 0.f;
-      for (int i = 0; i < d; ++i) kq = fmaf(qkv[t * C + kvh * d + i], qkv[t * C + (G + kvh) * d + i], kq);
-      skq[lane] = kq;
-      sbeta[lane] = sigmoidf_(ld(b_raw + t * ld_b + h));
     }
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
-      const size_t t = (size_t)(first + t0 + tt);
-      const float v = live ? qkv[t * C + 2 * G * d + h * dv + e] : 0.f;
-      float dk = 0.f, dq = 0.f;
+      float dk = 0.f;
+#pragma unroll
+      for (int i = 0; i < DP; ++i) dk = fmaf(S[i], sgk[tt][i], dk);
+      const float u = sbeta[tt] * (sv[tt][lane] - dk);
+      float o = 0.f;
 #pragma unroll
       for (int i = 0; i < DP; ++i) {
-        dk = fmaf(S[i], sgk[tt][i], dk);
-        dq = fmaf(S[i], sgq[tt][i], dq);
+        S[i] = fmaf(sk[tt][i], u, sg[tt][i] * S[i]);
+        if (MODE != 1) o = fmaf(S[i], sq[tt][i], o);
       }
-      const float u = sbeta[tt] * (v - dk);
-#pragma unroll
-      for (int i = 0; i < DP; ++i) S[i] = fmaf(sk[tt][i], u, sg[tt][i] * S[i]);
-      if (live) out[t * (size_t)(H * dv) + h * dv + e] = fmaf(u, skq[tt], dq);
+      if (MODE != 1 && live) out[(size_t)(first + t0 + tt) * (size_t)(H * dv) + h * dv + e] = o;
     }
   }
-  if (live) {
+  if (!live) return;
+  if (MODE == 1) {
+    float* dst = scratch + ((size_t)blockIdx.z * H + h) * d * (size_t)(dv + d);
+#pragma unroll
+    for (int i = 0; i < DP; ++i)
+      if (i < d) dst[(size_t)i * (dv + d) + e] = S[i];
+  } else if (last_chunk) {
+    float* Srow = state + ((size_t)slots[b] * H + h) * d * dv;
 #pragma unroll
     for (int i = 0; i < DP; ++i)
       if (i < d) Srow[(size_t)i * dv + e] = S[i];
+  }
+}
+
+// Walks the chunks of a request: start[first chunk] = the request's state (zero for a fresh one), start[c + 1] = P_c start[c] + L_c.
+// Workgroup = (column block of 64, head, request); a thread owns column e.  The current start state sits in LDS (one column per
+// thread), P_c comes through LDS sixteen rows at a time, and every new row goes straight to start[c + 1], from where the thread
+// reads its own column back for the next chunk.
+template <int DP>
+__global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict__ state, const float* __restrict__ scratch,
+                                                        float* __restrict__ start, const int* __restrict__ cu_q,
+                                                        const int* __restrict__ seq_lens, const int* __restrict__ slots,
+                                                        const int* __restrict__ item_first, int H, int d, int dv) {
+  extern __shared__ __attribute__((aligned(16))) float scan_lds[];
+  float* Sc = scan_lds;            // [DP][64]
+  float* P = scan_lds + DP * 64;   // [16][DP]
+  const int b = blockIdx.z, h = blockIdx.y, e = blockIdx.x * 64 + threadIdx.x, lane = threadIdx.x;
+  const int c0 = item_first[b], c1 = item_first[b + 1];
+  if (c1 <= c0) return;
+  const bool live = e < dv;
+  const bool fresh = seq_lens[b] == cu_q[b + 1] - cu_q[b];
+  const float* Srow = state + ((size_t)slots[b] * H + h) * d * dv;
+  float* dst = start + ((size_t)c0 * H + h) * d * dv;
+  for (int i = 0; i < DP; ++i) {
+    const float v = (!fresh && live && i < d) ? Srow[(size_t)i * dv + e] : 0.f;
+    Sc[i * 64 + lane] = v;
+    if (live && i < d) dst[(size_t)i * dv + e] = v;
+  }
+  for (int c = c0; c + 1 < c1; ++c) {
+    const float* LP = scratch + ((size_t)c * H + h) * d * (size_t)(dv + d);
+    dst = start + ((size_t)(c + 1) * H + h) * d * dv;
+    for (int i0 = 0; i0 < d; i0 += 16) {
+      __syncthreads();
+      for (int idx = lane; idx < 16 * DP; idx += 64) {
+        const int r = idx / DP, j = idx - r * DP;
+        P[idx] = (i0 + r < d && j < d) ? LP[(size_t)(i0 + r) * (dv + d) + dv + j] : 0.f;
+      }
+      __syncthreads();
+      float acc[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = (live && i0 + r < d) ? LP[(size_t)(i0 + r) * (dv + d) + e] : 0.f;
+      for (int j = 0; j < DP; j += 4) {
+        const float s0 = Sc[j * 64 + lane], s1 = Sc[(j + 1) * 64 + lane], s2 = Sc[(j + 2) * 64 + lane], s3 = Sc[(j + 3) * 64 + lane];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float4 p = *reinterpret_cast<const float4*>(P + r * DP + j);
+          acc[r] = fmaf(p.x, s0, fmaf(p.y, s1, fmaf(p.z, s2, fmaf(p.w, s3, acc[r]))));
+        }
+      }
+      if (live) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (i0 + r < d) dst[(size_t)(i0 + r) * dv + e] = acc[r];
+      }
+    }
+    __syncthreads();
+    for (int i = 0; i < d; ++i) Sc[i * 64 + lane] = live ? dst[(size_t)i * dv + e] : 0.f;
   }
 }
 
@@ -737,23 +835,38 @@ int msgl_mix_short_conv(float* out, const void* src, int64_t ld_src, const void*
 
 int msgl_mix_delta_rule(float* out, const float* qkv, float* state, const void* b_raw, int64_t ld_b, const void* a_raw, int64_t ld_a,
                         int per_channel, const float* rate, const float* dt_bias, const int* cu_q, const int* seq_lens, const int* slots,
-                        int batch, int H, int G, int d, int dv, int dtype, void* stream) {
+                        int batch, int H, int G, int d, int dv, int dtype, int n_items, const int* items, const int* item_first,
+                        float* scratch, void* stream) {
   MIX_REQUIRE(out && qkv && state && b_raw && a_raw && rate && dt_bias && cu_q && seq_lens && slots && dtype_ok(dtype),
               "delta_rule: null pointer / dtype");
   MIX_REQUIRE(batch >= 0 && H >= 1 && G >= 1 && H % G == 0 && d >= 1 && d <= 256 && dv >= 1, "delta_rule: bad sizes H %d G %d d %d dv %d", H,
               G, d, dv);
   MIX_REQUIRE(ld_b >= H && ld_a >= (per_channel ? H * d : H), "delta_rule: rows shorter than their heads");
+  MIX_REQUIRE(n_items >= 0 && (n_items == 0 || (items && item_first && scratch)), "delta_rule: chunks without their lists / scratch");
   if (batch == 0) return MSGL_MIX_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid((dv + 63) / 64, H, batch);
-#define DR_LAUNCH(DP, CH)                                                                                                             \
-  DISPATCH_T(dtype, hipLaunchKernelGGL((delta_rule_kernel<T, DP, CH>), grid, dim3(64), 0, s, out, qkv, state, cp<T>(b_raw), ld_b,     \
-                                       cp<T>(a_raw), ld_a, rate, dt_bias, cu_q, seq_lens, slots, H, G, d, dv);)
-#define DR_CASE(DP)            \
-  if (per_channel) {           \
-    DR_LAUNCH(DP, true)        \
-  } else {                     \
-    DR_LAUNCH(DP, false)       \
+  float* start = scratch ? scratch + (size_t)n_items * H * d * (size_t)(dv + d) : nullptr;  // [n_items, H, d, dv] after (L | P)
+#define DR_LAUNCH(DP, CH, MODE, GRID)                                                                                                  \
+  DISPATCH_T(dtype, hipLaunchKernelGGL((delta_rule_kernel<T, DP, CH, MODE>), GRID, dim3(64), 0, s, out, qkv, state, cp<T>(b_raw), ld_b, \
+                                       cp<T>(a_raw), ld_a, rate, dt_bias, cu_q, seq_lens, slots, H, G, d, dv, items, item_first,       \
+                                       scratch, start);)
+#define DR_RUN(DP, CH)                                                                                                         \
+  if (n_items == 0) {                                                                                                          \
+    DR_LAUNCH(DP, CH, 0, dim3((dv + 63) / 64, H, batch))                                                                       \
+  } else {                                                                                                                     \
+    DR_LAUNCH(DP, CH, 1, dim3((dv + d + 63) / 64, H, n_items))                                                                 \
+    MIX_LAUNCHED("delta_rule (chunk transitions)");                                                                            \
+    MIX_REQUIRE(ensure_lds((const void*)delta_scan_kernel<DP>, (size_t)(DP * 80) * 4) == 0, "delta_rule: scan LDS");           \
+    hipLaunchKernelGGL((delta_scan_kernel<DP>), dim3((dv + 63) / 64, H, batch), dim3(64), (size_t)(DP * 80) * 4, s, state,     \
+                       scratch, start, cu_q, seq_lens, slots, item_first, H, d, dv);                                           \
+    MIX_LAUNCHED("delta_rule (scan)");                                                                                         \
+    DR_LAUNCH(DP, CH, 2, dim3((dv + 63) / 64, H, n_items))                                                                     \
+  }
+#define DR_CASE(DP)     \
+  if (per_channel) {    \
+    DR_RUN(DP, true)    \
+  } else {              \
+    DR_RUN(DP, false)   \
   }
   if (d <= 16) {
     DR_CASE(16)
@@ -771,6 +884,7 @@ int msgl_mix_delta_rule(float* out, const float* qkv, float* state, const void* 
     DR_CASE(256)
   }
 #undef DR_CASE
+#undef DR_RUN
 #undef DR_LAUNCH
   MIX_LAUNCHED("delta_rule");
   return MSGL_MIX_OK;

@@ -530,7 +530,7 @@ class HybridDecoder:
             a_raw, gate, act = proj[:, C + H: C + 2 * H], proj[:, C + 2 * H: C + 2 * H + H * dv], mixops.GATE_SILU
         o = torch.empty((T, H * dv), dtype=torch.float32, device=h.device)
         mixops.delta_rule(o, qkv, kv.state(i), b_raw, a_raw, s.kind == "channel_delta", L.rate, L.dt_bias, md.cu_seqlens_q, md.seq_lens,
-                          md.req_rows, md.batch, G)
+                          md.req_rows, md.batch, G, chunks=getattr(md, "delta_chunks", None))
         return mixops.linear(mixops.head_gated_norm(o, gate, L.out_norm, self.cfg.rms_norm_eps, H, dv, act), L.o)
 
     def _gated_experts(self, L: _Layer, h: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:

@@ -399,9 +399,10 @@ def short_conv(src: torch.Tensor, C: int, taps: torch.Tensor, state: Optional[to
 
 def delta_rule(out: torch.Tensor, qkv: torch.Tensor, state: torch.Tensor, b_raw: torch.Tensor, a_raw: torch.Tensor, per_channel: bool,
                rate: torch.Tensor, dt_bias: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor, slots: torch.Tensor, batch: int,
-               G: int) -> None:
+               G: int, chunks=None) -> None:
     """state: fp32 [slots, H, d, dv]; qkv: fp32 rows [q G*d | k G*d | v H*dv]; b_raw [T, H], a_raw [T, H] or [T, H*d] in the model
-    dtype (views with a row stride are fine); rate = -exp(A_log) and dt_bias in fp32."""
+    dtype (views with a row stride are fine); rate = -exp(A_log) and dt_bias in fp32.  chunks = (items int32 [n, 3], item_first
+    int32 [batch + 1], n) cuts long portions into pieces that run in parallel (see include/msgl_mix.h)."""
     _dev(out, qkv, state, b_raw, a_raw, rate, dt_bias, cu_q, seq_lens, slots)
     _, H, d, dv = state.shape
     T = qkv.shape[0]
@@ -410,10 +411,18 @@ def delta_rule(out: torch.Tensor, qkv: torch.Tensor, state: torch.Tensor, b_raw:
     assert qkv.shape == (T, 2 * G * d + H * dv) and out.dtype == torch.float32 and out.is_contiguous() and out.shape == (T, H * dv)
     assert b_raw.stride(1) == 1 and a_raw.stride(1) == 1 and b_raw.shape == (T, H) and a_raw.shape == (T, na) and a_raw.dtype == b_raw.dtype
     assert rate.dtype == torch.float32 and rate.shape == (H,) and dt_bias.dtype == torch.float32 and dt_bias.shape == (na,)
+    items = first = scratch = None
+    n_items = 0
+    if chunks is not None:
+        items, first, n_items = chunks
+        _dev(items, first)
+        assert items.numel() == 3 * n_items and first.numel() == batch + 1
+        scratch = torch.empty(n_items * H * d * (2 * dv + d), dtype=torch.float32, device=out.device)
     check_mix(mix_lib().msgl_mix_delta_rule(
         out.data_ptr(), qkv.data_ptr(), state.data_ptr(), b_raw.data_ptr(), b_raw.stride(0), a_raw.data_ptr(), a_raw.stride(0),
         int(per_channel), rate.data_ptr(), dt_bias.data_ptr(), _i32(cu_q).data_ptr(), _i32(seq_lens).data_ptr(), _i32(slots).data_ptr(),
-        batch, H, G, d, dv, _code(b_raw), _stream()), "delta_rule")
+        batch, H, G, d, dv, _code(b_raw), n_items, _p(None if items is None else _i32(items)),
+        _p(None if first is None else _i32(first)), _p(scratch), _stream()), "delta_rule")
 
 
 def head_gated_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, H: int, dv: int, gate_act: int) -> torch.Tensor:

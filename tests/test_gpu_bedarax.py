@@ -205,9 +205,11 @@ def test_window_edges_one_key_stands_out(dev, dtype, window, splits):
                 assert float((got[outside] - want).abs().max()) > 0.05 * float(want.abs().max())
 
 
-def test_delta_rule_state_slots_and_cuts(dev):
+@pytest.mark.parametrize("chunk", [0, 1, 5], ids=["whole", "chunks-of-1", "chunks-of-5"])
+def test_delta_rule_state_slots_and_cuts(dev, chunk):
     """The recurrence kernel alone: two requests in one launch on state rows that hold garbage, then continued in a second
-    launch; per-head and per-channel decays, grouped keys.  Against the token loop of the restatement."""
+    launch; per-head and per-channel decays, grouped keys; whole portions, and portions cut into pieces that run in parallel
+    and are joined by the scan.  Against the token loop of the restatement."""
     from mini_sglang_amd import mixops
 
     for per_channel in (False, True):
@@ -234,9 +236,17 @@ def test_delta_rule_state_slots_and_cuts(dev):
             a_raw = torch.cat([seq[b]["a"][s:e] for b, (s, e) in cuts.items()]).float().to(dev)
             cu = torch.tensor([0, cuts[0][1] - cuts[0][0], qkv.shape[0]], dtype=torch.int32, device=dev)
             out = torch.empty((qkv.shape[0], H * dv), dtype=torch.float32, device=dev)
+            chunks = None
+            if chunk:
+                items, firsts = [], [0]
+                for bb, (s0, e0) in cuts.items():
+                    items += [[bb, c, min(c + chunk, e0 - s0)] for c in range(0, e0 - s0, chunk)]
+                    firsts.append(len(items))
+                chunks = (torch.tensor(items, dtype=torch.int32, device=dev).view(-1), torch.tensor(firsts, dtype=torch.int32, device=dev),
+                          len(items))
             mixops.delta_rule(out, qkv, state, b_raw, a_raw, per_channel, rate.float().to(dev), dtb.float().to(dev), cu,
                               torch.tensor([cuts[0][1], cuts[1][1]], dtype=torch.int32, device=dev),
-                              torch.tensor([2, 0], dtype=torch.int32, device=dev), 2, G)
+                              torch.tensor([2, 0], dtype=torch.int32, device=dev), 2, G, chunks=chunks)
             outs[0].append(out[: cu[1]].cpu())
             outs[1].append(out[cu[1]:].cpu())
         for b, n in enumerate(lens):
@@ -270,6 +280,18 @@ def test_portions_fp32(sizes):
     eng_state = engine_for(FULL, torch.float32)
     toks = tokens_of(131, FULL["vocab"], 6)
     check(eng_state, FULL, alone("a", toks, sizes), {"a": toks}, FP32_TOL)
+
+
+def test_long_portions_run_as_parallel_chunks_fp32():
+    """Portions long enough for the delta-rule layers to cut them into pieces (states joined by a scan): first a long portion
+    from position 0, then a single token, then a long portion that continues from a carried state, beside a short request;
+    lengths off the piece size."""
+    eng_state = engine_for(FULL, torch.float32, max_tokens=2048)
+    a, b = tokens_of(1200, FULL["vocab"], 30), tokens_of(6, FULL["vocab"], 31)
+    steps = [[("a", a[:560], False)], [("a", a[560:561], False), ("b", b[:5], False)], [("b", b[5:], True), ("a", a[561:], True)]]
+    got = check(eng_state, FULL, steps, {"a": a, "b": b}, FP32_TOL)
+    whole = replay(eng_state[0], alone("a", a, [257, 443]))["a"]
+    assert rel(got["a"], whole) < 2e-5
 
 
 def test_long_decoding_fp32():

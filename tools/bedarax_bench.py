@@ -117,10 +117,16 @@ def kernel_rooflines(name: str, prompt: int, batch: int, device) -> dict:
         state = torch.zeros(reqs, H, D, D, dtype=torch.float32, device=device)
         rate = -torch.rand(H, device=device)
         od = torch.empty(T, H * D, dtype=torch.float32, device=device)
+        dchunks = None
+        if q_len >= 512:  # what the engine's metadata does for long portions: pieces of 256 tokens in parallel
+            n = -(-q_len // 256)
+            items = i32([[b, c * 256, min((c + 1) * 256, q_len)] for b in range(reqs) for c in range(n)]).view(-1)
+            dchunks = (items, i32([b * n for b in range(reqs + 1)]), reqs * n)
         for label, chan in (("delta_rule", False), ("channel_delta_rule", True)):
             a_raw = rnd(T, H * D if chan else H)
             dtb = torch.zeros(H * D if chan else H, dtype=torch.float32, device=device)
-            us = _time_us(lambda: mixops.delta_rule(od, qkv, state, proj[:, C: C + H], a_raw, chan, rate, dtb, cu, seq, rows, reqs, H))
+            us = _time_us(lambda: mixops.delta_rule(od, qkv, state, proj[:, C: C + H], a_raw, chan, rate, dtb, cu, seq, rows, reqs, H,
+                                                    chunks=dchunks))
             byts = 2 * reqs * H * D * D * 4 + T * C * 4 + T * H * D * 4
             out[f"{phase}.{label}"] = _entry(us, 8.0 * T * H * D * D, byts, VALU_TFLOPS)
         lq = rnd(T, 4 * H * D, scale=0.5)
