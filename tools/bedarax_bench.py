@@ -93,7 +93,9 @@ def kernel_rooflines(name: str, prompt: int, batch: int, device) -> dict:
         kc, vc = rnd(slots, G * D, scale=0.3), rnd(slots, G * D)
         talk = torch.eye(H, device=device) + 0.05 * torch.randn(H, H, device=device)
         o = torch.empty(T, H * D, dtype=bf, device=device)
-        us = _time_us(lambda: mixops.window_attn(o, src, H * D, kc, vc, table, rows, seq, cu, reqs, H, G, D, D, window, D ** -0.5, talk))
+        wsplits = mixops.window_attn_splits(reqs, T, window, ctx)
+        us = _time_us(lambda: mixops.window_attn(o, src, H * D, kc, vc, table, rows, seq, cu, reqs, H, G, D, D, window, D ** -0.5, talk,
+                                                 splits=wsplits))
         first = ctx - q_len
         pairs = reqs * sum(min(first + i + 1, window) for i in range(q_len))
         keys_read = reqs * min(ctx, window + q_len - 1)
