@@ -574,6 +574,33 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(float* __restrict__ out,
       sg[tt][i] = g;
     }
     __syncthreads();
+    if (d == DP) {
+      // q and k of a token are the same for every lane: read straight from the fp32 rows through uniform addresses (the scalar
+      // unit's loads), so that the LDS carries only what had to be computed (the per-channel decays) -- LDS reads bound this loop
+      for (int tt = 0; tt < nt; ++tt) {
+        const float* __restrict__ qp = qkv + (size_t)(first + t0 + tt) * C + kvh * DP;
+        const float* __restrict__ kp = qkv + (size_t)(first + t0 + tt) * C + (G + kvh) * DP;
+        float dk = 0.f;
+        if (CHANNEL) {
+#pragma unroll
+          for (int i = 0; i < DP; ++i) dk = fmaf(S[i], sgk[tt][i], dk);
+        } else {
+#pragma unroll
+          for (int i = 0; i < DP; ++i) dk = fmaf(S[i], kp[i], dk);
+          dk *= sdec[tt];
+        }
+        const float u = sbeta[tt] * (sv[tt][lane] - dk);
+        const float gs = sdec[tt];
+        float o = 0.f;
+#pragma unroll
+        for (int i = 0; i < DP; ++i) {
+          S[i] = fmaf(kp[i], u, (CHANNEL ? sg[tt][i] : gs) * S[i]);
+          if (MODE != 1) o = fmaf(S[i], qp[i], o);
+        }
+        if (MODE != 1 && live) out[(size_t)(first + t0 + tt) * (size_t)(H * dv) + h * dv + e] = o;
+      }
+      continue;
+    }
     for (int tt = 0; tt < nt; ++tt) {
       float dk = 0.f;
 #pragma unroll
