@@ -630,58 +630,74 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(float* __restrict__ out,
 }
 
 // Walks the chunks of a request: start[first chunk] = the request's state (zero for a fresh one), start[c + 1] = P_c start[c] + L_c.
-// Workgroup = (column block of 64, head, request); a thread owns column e.  The current start state sits in LDS (one column per
-// thread), P_c comes through LDS sixteen rows at a time, and every new row goes straight to start[c + 1], from where the thread
-// reads its own column back for the next chunk.
+// Workgroup = (column block of 64, head, request), NW waves; a lane owns column e, the waves share the rows: wave w computes rows
+// 16 w .. 16 w + 15 of every block of 16 NW rows from its own LDS tile of P_c.  The current start state sits in LDS (one column per
+// lane), the new one is built in a second LDS buffer and written to start[c + 1] on the way; the buffers swap per chunk.
 template <int DP>
-__global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict__ state, const float* __restrict__ scratch,
-                                                        float* __restrict__ start, const int* __restrict__ cu_q,
-                                                        const int* __restrict__ seq_lens, const int* __restrict__ slots,
-                                                        const int* __restrict__ item_first, int H, int d, int dv) {
+struct ScanShape {
+  static constexpr int NW = DP > 128 ? 2 : 4;   // waves
+  static constexpr int PR = DP > 128 ? 8 : 16;  // rows of P per wave and block
+  static constexpr size_t lds_bytes = (size_t)(2 * DP * 64 + NW * PR * DP) * sizeof(float);
+};
+
+template <int DP>
+__global__ __launch_bounds__(ScanShape<DP>::NW * 64) void delta_scan_kernel(const float* __restrict__ state,
+                                                                            const float* __restrict__ scratch, float* __restrict__ start,
+                                                                            const int* __restrict__ cu_q, const int* __restrict__ seq_lens,
+                                                                            const int* __restrict__ slots,
+                                                                            const int* __restrict__ item_first, int H, int d, int dv) {
+  constexpr int NW = ScanShape<DP>::NW, PR = ScanShape<DP>::PR;
   extern __shared__ __attribute__((aligned(16))) float scan_lds[];
-  float* Sc = scan_lds;            // [DP][64]
-  float* P = scan_lds + DP * 64;   // [16][DP]
-  const int b = blockIdx.z, h = blockIdx.y, e = blockIdx.x * 64 + threadIdx.x, lane = threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float* cur = scan_lds;                              // [DP][64]
+  float* nxt = scan_lds + DP * 64;                    // [DP][64]
+  float* P = scan_lds + 2 * DP * 64 + wave * PR * DP; // [PR][DP], this wave's
+  const int b = blockIdx.z, h = blockIdx.y, e = blockIdx.x * 64 + lane;
   const int c0 = item_first[b], c1 = item_first[b + 1];
   if (c1 <= c0) return;
   const bool live = e < dv;
   const bool fresh = seq_lens[b] == cu_q[b + 1] - cu_q[b];
   const float* Srow = state + ((size_t)slots[b] * H + h) * d * dv;
   float* dst = start + ((size_t)c0 * H + h) * d * dv;
-  for (int i = 0; i < DP; ++i) {
+  for (int i = wave; i < DP; i += NW) {
     const float v = (!fresh && live && i < d) ? Srow[(size_t)i * dv + e] : 0.f;
-    Sc[i * 64 + lane] = v;
+    cur[i * 64 + lane] = v;
+    nxt[i * 64 + lane] = 0.f;
     if (live && i < d) dst[(size_t)i * dv + e] = v;
   }
   for (int c = c0; c + 1 < c1; ++c) {
     const float* LP = scratch + ((size_t)c * H + h) * d * (size_t)(dv + d);
     dst = start + ((size_t)(c + 1) * H + h) * d * dv;
-    for (int i0 = 0; i0 < d; i0 += 16) {
-      __syncthreads();
-      for (int idx = lane; idx < 16 * DP; idx += 64) {
+    for (int blk = 0; blk < d; blk += NW * PR) {
+      const int i0 = blk + wave * PR;
+      __syncthreads();  // the state of this chunk is complete (first block) / the wave's tile is free again
+      for (int idx = lane; idx < PR * DP; idx += 64) {
         const int r = idx / DP, j = idx - r * DP;
         P[idx] = (i0 + r < d && j < d) ? LP[(size_t)(i0 + r) * (dv + d) + dv + j] : 0.f;
       }
       __syncthreads();
-      float acc[16];
+      float acc[PR];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = (live && i0 + r < d) ? LP[(size_t)(i0 + r) * (dv + d) + e] : 0.f;
+      for (int r = 0; r < PR; ++r) acc[r] = (live && i0 + r < d) ? LP[(size_t)(i0 + r) * (dv + d) + e] : 0.f;
       for (int j = 0; j < DP; j += 4) {
-        const float s0 = Sc[j * 64 + lane], s1 = Sc[(j + 1) * 64 + lane], s2 = Sc[(j + 2) * 64 + lane], s3 = Sc[(j + 3) * 64 + lane];
+        const float s0 = cur[j * 64 + lane], s1 = cur[(j + 1) * 64 + lane], s2 = cur[(j + 2) * 64 + lane], s3 = cur[(j + 3) * 64 + lane];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
+        for (int r = 0; r < PR; ++r) {
           const float4 p = *reinterpret_cast<const float4*>(P + r * DP + j);
           acc[r] = fmaf(p.x, s0, fmaf(p.y, s1, fmaf(p.z, s2, fmaf(p.w, s3, acc[r]))));
         }
       }
-      if (live) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if (i0 + r < d) dst[(size_t)(i0 + r) * dv + e] = acc[r];
+      for (int r = 0; r < PR; ++r) {
+        if (i0 + r < d) {
+          nxt[(i0 + r) * 64 + lane] = acc[r];
+          if (live) dst[(size_t)(i0 + r) * dv + e] = acc[r];
+        }
       }
     }
-    __syncthreads();
-    for (int i = 0; i < d; ++i) Sc[i * 64 + lane] = live ? dst[(size_t)i * dv + e] : 0.f;
+    float* t = cur;
+    cur = nxt;
+    nxt = t;
   }
 }
 
@@ -883,9 +899,9 @@ int msgl_mix_delta_rule(float* out, const float* qkv, float* state, const void* 
   } else {                                                                                                                     \
     DR_LAUNCH(DP, CH, 1, dim3((dv + d + 63) / 64, H, n_items))                                                                 \
     MIX_LAUNCHED("delta_rule (chunk transitions)");                                                                            \
-    MIX_REQUIRE(ensure_lds((const void*)delta_scan_kernel<DP>, (size_t)(DP * 80) * 4) == 0, "delta_rule: scan LDS");           \
-    hipLaunchKernelGGL((delta_scan_kernel<DP>), dim3((dv + 63) / 64, H, batch), dim3(64), (size_t)(DP * 80) * 4, s, state,     \
-                       scratch, start, cu_q, seq_lens, slots, item_first, H, d, dv);                                           \
+    MIX_REQUIRE(ensure_lds((const void*)delta_scan_kernel<DP>, ScanShape<DP>::lds_bytes) == 0, "delta_rule: scan LDS");         \
+    hipLaunchKernelGGL((delta_scan_kernel<DP>), dim3((dv + 63) / 64, H, batch), dim3(ScanShape<DP>::NW * 64),                  \
+                       ScanShape<DP>::lds_bytes, s, state, scratch, start, cu_q, seq_lens, slots, item_first, H, d, dv);       \
     MIX_LAUNCHED("delta_rule (scan)");                                                                                         \
     DR_LAUNCH(DP, CH, 2, dim3((dv + 63) / 64, H, n_items))                                                                     \
   }
