@@ -320,7 +320,7 @@ class HybridDecoder:
         return self.weight_bytes()
 
     def load_state(self, state: Dict[str, torch.Tensor]) -> None:
-        """Overwrite the seeded weights with a checkpoint's tensors (names as in its TENSORS listing: 'embed', 'final.norm',
+        """Overwrite the seeded weights with a checkpoint's tensors (checkpoint names: 'embed', 'final.norm',
         'l<i>.norm1', 'l<i>.mix.<name>', 'l<i>.mlp.e<j>.up' ...), merging what one launch reads together: q | dkv, q | k | v | g,
         the experts of a layer stacked, W_uk split per head and transposed."""
         cfg = self.cfg
