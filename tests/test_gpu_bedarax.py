@@ -97,12 +97,22 @@ def check(eng_state, cfg_json, steps, seqs, tol, allow=0.0):
     delta(), delta(heads=3, kv_heads=3, dim=20, vdim=70, conv=4), delta(heads=2, kv_heads=1, dim=40, vdim=12, conv=1),
     delta(heads=1, kv_heads=1, dim=72, vdim=8, conv=6),
     delta(channel=True), delta(channel=True, heads=2, kv_heads=2, dim=36, vdim=80, conv=5),
+    delta(heads=2, kv_heads=1, dim=64, vdim=16), delta(channel=True, heads=1, kv_heads=1, dim=128, vdim=72, conv=2),
+    delta(heads=1, kv_heads=1, dim=192, vdim=8, conv=2),
 ], ids=["attention-grouped", "attention-odd-sizes", "attention-no-window", "attention-window-one", "attention-window-at-tile",
-        "delta-grouped", "delta-wide-v", "delta-one-tap", "delta-wide-key", "channel-delta-grouped", "channel-delta-wide"])
+        "delta-grouped", "delta-wide-v", "delta-one-tap", "delta-wide-key", "channel-delta-grouped", "channel-delta-wide",
+        "delta-key-64", "channel-delta-key-128", "delta-key-192"])
 def test_mixer_alone_fp32(layer):
     cfg = config([layer])
     toks = tokens_of(70, cfg["vocab"], 1)
     check(engine_for(cfg, torch.float32), cfg, alone("a", toks, [70]), {"a": toks}, FP32_TOL)
+
+
+def test_attention_many_wide_heads_bf16():
+    """Twelve heads of 128: the 8-token query tile needs more LDS than a kernel gets by default; 16-bit keys and values."""
+    cfg = config([att(heads=12, kv_heads=4, dim=128, vdim=32, window=40, scale=0.09)], width=64)
+    toks = tokens_of(150, cfg["vocab"], 12)
+    check(engine_for(cfg, torch.bfloat16), cfg, alone("a", toks, [100, 1, 1, 5, 43]), {"a": toks}, BF16_TOL)
 
 
 @pytest.mark.parametrize("mlp", [dense(), dense(ff=300), moe(), moe(experts=4, top=1), moe(experts=3, top=3, ff=8), moe(experts=70, top=6, ff=16)],
@@ -430,3 +440,9 @@ def test_trace_command_line(tmp_path):
     got2 = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(2, -1)).double()
     assert rel(got0, ra[[0, 29]]) < FP32_TOL and rel(got1, ra[[30]]) < FP32_TOL
     assert rel(got2, torch.stack([ra[44], rb[8]])) < FP32_TOL
+    # the same folder through `generate`: greedy tokens in 16 bits, in range and of the asked length
+    pr = subprocess.run([sys.executable, "-m", "mini_sglang_amd.cli", "generate", "--model", str(mdir), "--prompt", "5,17,3", "--prompt",
+                         ",".join(map(str, a[:20])), "--max-tokens", "6"], cwd=str(root), text=True, capture_output=True, timeout=110)
+    assert pr.returncode == 0, pr.stderr[-2000:]
+    outs = [json.loads(ln)["output"] for ln in pr.stdout.splitlines() if ln.startswith("{")]
+    assert len(outs) == 2 and all(len(o) == 6 and all(0 <= t < cfg["vocab"] for t in o) for o in outs)
