@@ -142,14 +142,85 @@ __global__ __launch_bounds__(256) void prenorm_kernel(const float* __restrict__ 
   float* sc = red + 4;
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int e = wave; e < E; e += 4) {
-    float acc = 0.f;
-    for (int i = lane; i < W; i += 64) acc = fmaf(srow[i], ld(router + (size_t)e * W + i), acc);
-    acc = wave_sum(acc);
-    if (lane == 0) sc[e] = acc + (bias ? ld(bias + e) : 0.f);
+  // a wave takes experts wave, wave + 4, ...; up to kRouteAcc of them at once, so that one pass over the row keeps that many
+  // independent weight loads in flight per lane (16-byte loads where the row allows; element order per expert fixed)
+  constexpr int kRouteAcc = 8;
+  const bool wide = (W & 7) == 0 && ((uintptr_t)router & 15u) == 0;
+  for (int e0 = wave; e0 < E; e0 += 4 * kRouteAcc) {
+    float acc[kRouteAcc];
+#pragma unroll
+    for (int a = 0; a < kRouteAcc; ++a) acc[a] = 0.f;
+    if (wide) {
+      for (int i = lane * 8; i < W; i += 512) {
+        float hv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) hv[u] = srow[i + u];
+#pragma unroll
+        for (int a = 0; a < kRouteAcc; ++a) {
+          const int e = e0 + 4 * a;
+          if (e < E) {
+            float wv[8];
+            read8(router + (size_t)e * W + i, wv);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc[a] = fmaf(hv[u], wv[u], acc[a]);
+          }
+        }
+      }
+    } else {
+      for (int i = lane; i < W; i += 64) {
+        const float hv = srow[i];
+#pragma unroll
+        for (int a = 0; a < kRouteAcc; ++a) {
+          const int e = e0 + 4 * a;
+          if (e < E) acc[a] = fmaf(hv, ld(router + (size_t)e * W + i), acc[a]);
+        }
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < kRouteAcc; ++a) {
+      const int e = e0 + 4 * a;
+      const float v = wave_sum(acc[a]);
+      if (e < E && lane == 0) sc[e] = v + (bias ? ld(bias + e) : 0.f);
+    }
   }
   __syncthreads();
-  if (threadIdx.x == 0) select_top_logits(sc, 1, E, top, ids + (size_t)t * top, wts + (size_t)t * top);
+  if (wave != 0) return;
+  // the `top` largest logits by the 64 lanes of one wave (a lane owns experts lane, lane + 64, ...; ties: lowest index)
+  float first = 0.f, tot = 0.f, mine = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float bv = -INFINITY;
+    int best = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float v = sc[e];
+      if (v > bv) {
+        bv = v;
+        best = e;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(best, o, 64);
+      if (ov > bv || (ov == bv && oi < best)) {
+        bv = ov;
+        best = oi;
+      }
+    }
+    if (k == 0) first = bv;
+    const float p = expf(bv - first);
+    tot += p;
+    if (lane == k % 64) mine = p;  // lane k keeps the k-th weight (top <= 64 per pass of this loop is all a model has)
+    if (lane == 0) {
+      ids[(size_t)t * top + k] = best;
+      sc[best] = -INFINITY;
+    }
+    if (k % 64 == 63 || k == top - 1) {
+      // flush the weights gathered so far (unnormalised; the division follows once the total is known)
+      const int base = k - (k % 64);
+      if (base + lane <= k) wts[(size_t)t * top + base + lane] = mine;
+    }
+  }
+  for (int k = lane; k < top; k += 64) wts[(size_t)t * top + k] /= tot;
 }
 
 // ------------------------------------------------------------------------------------------------ activations
@@ -404,26 +475,34 @@ __global__ __launch_bounds__(256) void window_attn_kernel(T* __restrict__ out, f
     }
 }
 
-// Joins the key ranges of window_attn_kernel: one workgroup per token.
+// Joins the key ranges of window_attn_kernel: one workgroup per token.  The (m, l) pairs of all ranges and heads are folded once into
+// per-range factors exp(m_s - M) / L in LDS; every output element is then a short sum of independent loads.
 template <typename T>
 __global__ __launch_bounds__(256) void window_merge_kernel(T* __restrict__ out, const float* __restrict__ part_o,
                                                            const float* __restrict__ part_ml, const T* __restrict__ src, int64_t ld_src,
                                                            int g_off, int total_q, int H, int dv, int splits) {
+  extern __shared__ float fac[];  // [splits][H]
   const size_t t = blockIdx.x;
   const int no = H * dv;
-  for (int o = threadIdx.x; o < no; o += 256) {
-    const int h = o / dv;
+  for (int h = threadIdx.x; h < H; h += 256) {
     float m = -INFINITY;
     for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(((size_t)s * total_q + t) * H + h) * 2]);
-    float l = 0.f, v = 0.f;
+    float l = 0.f;
     for (int s = 0; s < splits; ++s) {
       const float* ml = part_ml + (((size_t)s * total_q + t) * H + h) * 2;
-      if (ml[0] == -INFINITY) continue;
-      const float f = expf(ml[0] - m);
+      const float f = ml[0] == -INFINITY ? 0.f : expf(ml[0] - m);
+      fac[s * H + h] = f;
       l = fmaf(ml[1], f, l);
-      v = fmaf(part_o[((size_t)s * total_q + t) * no + o], f, v);
     }
-    st(out + t * no + o, v / l * sigmoidf_(ld(src + t * ld_src + g_off + h)));
+    const float g = sigmoidf_(ld(src + t * ld_src + g_off + h)) / l;
+    for (int s = 0; s < splits; ++s) fac[s * H + h] *= g;
+  }
+  __syncthreads();
+  for (int o = threadIdx.x; o < no; o += 256) {
+    const int h = o / dv;
+    float v = 0.f;
+    for (int s = 0; s < splits; ++s) v = fmaf(part_o[((size_t)s * total_q + t) * no + o], fac[s * H + h], v);
+    st(out + t * no + o, v);
   }
 }
 
@@ -849,8 +928,8 @@ int msgl_mix_window_attn(void* out, const void* src, int64_t ld_src, int g_off, 
 #undef WA_LAUNCH
   MIX_LAUNCHED("window_attn");
   if (splits > 1) {
-    DISPATCH_T(dtype, hipLaunchKernelGGL(window_merge_kernel<T>, dim3(total_q), dim3(256), 0, s, mp<T>(out), part_o, part_ml, cp<T>(src),
-                                         ld_src, g_off, total_q, H, dv, splits);)
+    DISPATCH_T(dtype, hipLaunchKernelGGL(window_merge_kernel<T>, dim3(total_q), dim3(256), (size_t)splits * H * sizeof(float), s, mp<T>(out),
+                                         part_o, part_ml, cp<T>(src), ld_src, g_off, total_q, H, dv, splits);)
     MIX_LAUNCHED("window_attn (merge)");
   }
   return MSGL_MIX_OK;
