@@ -281,7 +281,12 @@ def test_baseline_config0_qwen3_0p6b_single_prompt_greedy(dev, page_size, new_to
                                              floor_cpu=cfloor, floor_cpu_agree=cfloor_same)
     dev_k = eng.kv_cache.pool[0].cpu().view(m.num_layers, slots, m.num_kv_heads, m.head_dim)
     for li in (0, m.num_layers // 2, m.num_layers - 1):  # one bf16 ulp of a K element of magnitude 4 is 3e-2
-        torch.testing.assert_close(dev_k[li][:-page_size].float(), kp[li][:-page_size].float(), atol=tol, rtol=tol)
+        # which projection kernel the timing-based plan search picks differs from run to run, and with it the rounding of single
+        # elements: a rotated element is a difference of two products of magnitude 4, so a handful of the 1 M elements may sit
+        # two ulps away (seen: 1 element at 6.6e-2); everything else within tol, nothing beyond twice tol
+        diff = (dev_k[li][:-page_size].float() - kp[li][:-page_size].float()).abs()
+        bound = tol + tol * kp[li][:-page_size].float().abs()
+        assert int((diff > bound).sum()) <= 4 and bool((diff <= 2 * bound).all()), (li, float(diff.max()))
     eng.shutdown()
 
 
