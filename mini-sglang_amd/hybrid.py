@@ -181,7 +181,8 @@ def bedarax_config(cfg: Dict[str, Any], shapes: Optional[Dict[str, Tuple[int, ..
             if kind == "channel_delta":
                 ra = int(shapes.get(f"l{i}.mix.a1", (max(d // 2, 8),))[0])
                 rg = int(shapes.get(f"l{i}.mix.g1", (max(d // 2, 8),))[0])
-            layers.append(LayerSpec(kind=kind, heads=H, kv_heads=G, dim=d, vdim=int(m["vdim"]), conv=int(m.get("conv", 1)),
+            taps = m.get("conv") or shapes.get(f"l{i}.mix.q.conv", (0, 1))[1]  # config.json, else the taps tensor's width
+            layers.append(LayerSpec(kind=kind, heads=H, kv_heads=G, dim=d, vdim=int(m["vdim"]), conv=int(taps),
                                     decay_rank=ra, gate_rank=rg, mlp=ff))
         else:
             raise ValueError(f"layer {i}: unknown mixer type {kind!r}")

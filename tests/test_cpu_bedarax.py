@@ -38,6 +38,9 @@ def test_config_reader_and_registry(tmp_path):
     assert (c.kind, c.conv, c.decay_rank, c.gate_rank) == ("channel_delta", 3, 5, 7) and isinstance(c.mlp, MoeSpec)
     assert c.mlp.gated and c.mlp.pick == "logits" and (c.mlp.experts, c.mlp.top, c.mlp.ff) == (5, 2, 12)
     assert d.mlp is None and d.recurrent and a2.window == 0
+    no_taps = _cfg()
+    del no_taps["layers"][2]["mixer"]["conv"]  # a size config.json leaves out comes from the tensor's shape
+    assert bedarax_config(no_taps, {"l2.mix.q.conv": (8, 5)}).layers[2].conv == 5 and bedarax_config(no_taps).layers[2].conv == 1
     bad = _cfg()
     bad["layers"][3]["mixer"]["vdim"] = 12  # value-mixing layers must agree
     with pytest.raises(ValueError):
